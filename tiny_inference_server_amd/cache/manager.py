@@ -79,6 +79,7 @@ class GroupSpec:
     n_kv_heads: int
     head_dim: int
     window: int                      # 0: every position stays readable
+    value_dim: int = 0               # channels of a value where they differ from head_dim (0: the same)
     keys: List[str] = field(default_factory=list)    # cache keys of the users, in plane order
 
 
@@ -98,8 +99,14 @@ class PageGroup:
             # [plane][page][key or value][kv head][slot in page][head size]; within a page and head the values
             # lie transposed, [head size][slot]. Zeroed once, as the reference does (block_table.py:40), though no
             # kernel needs it: slots that a row may not see are read, but replaced before any arithmetic
-            self.storage = torch.zeros((len(spec.keys), n_pages, 2, spec.n_kv_heads, page_size, spec.head_dim),
-                                       dtype=dtype, device=device)
+            if spec.value_dim and spec.value_dim != spec.head_dim:
+                # keys [kv head][slot][head size] of all heads, then values [kv head][value size][slot]: one line a page
+                self.storage = torch.zeros((len(spec.keys), n_pages,
+                                            spec.n_kv_heads * page_size * (spec.head_dim + spec.value_dim)),
+                                           dtype=dtype, device=device)
+            else:
+                self.storage = torch.zeros((len(spec.keys), n_pages, 2, spec.n_kv_heads, page_size, spec.head_dim),
+                                           dtype=dtype, device=device)
 
     def plane(self, key: str):
         return self.storage[self.plane_of[key]]
@@ -177,16 +184,18 @@ class CacheManager:
         n_slots = max_requests + (1 if spare_positions > 0 else 0)
         n_pages = n_pages + self._spare_pages
         self.dtype, self.device = dtype, device
-        specs: Dict[Tuple[int, int, int], GroupSpec] = {}
+        specs: Dict[Tuple[int, int, int, int], GroupSpec] = {}
         self.group_of: Dict[str, str] = {}
         self.states: Dict[str, Optional[torch.Tensor]] = {}
         self._state_needs: Dict[str, StateNeed] = {}
         for key, need in needs.items():
             if isinstance(need, PagedKvNeed):
-                geom = (need.n_kv_heads, need.head_dim, need.window)
+                vdim = need.value_dim if need.value_dim and need.value_dim != need.head_dim else 0
+                geom = (need.n_kv_heads, need.head_dim, need.window, vdim)
                 if geom not in specs:
-                    name = f"kv{need.n_kv_heads}x{need.head_dim}" + (f"w{need.window}" if need.window else "")
-                    specs[geom] = GroupSpec(name, need.n_kv_heads, need.head_dim, need.window)
+                    name = (f"kv{need.n_kv_heads}x{need.head_dim}" + (f"v{vdim}" if vdim else "") +
+                            (f"w{need.window}" if need.window else ""))
+                    specs[geom] = GroupSpec(name, need.n_kv_heads, need.head_dim, need.window, vdim)
                 specs[geom].keys.append(key)
                 self.group_of[key] = specs[geom].name
             elif isinstance(need, StateNeed):
@@ -280,13 +289,14 @@ class CacheManager:
         """Bytes that one more page costs: every group gets as many pages as every other, and a page of a group has
         a plane for each of the group's cache users (the reference's one geometry: block_table.py:34-38)."""
         elem = torch.empty(0, dtype=dtype).element_size()
-        return sum(2 * need.n_kv_heads * need.head_dim * page_size * elem
+        return sum(need.n_kv_heads * (need.head_dim + (need.value_dim or need.head_dim)) * page_size * elem
                    for need in needs.values() if isinstance(need, PagedKvNeed))
 
     def bytes_per_position(self) -> int:
         """Bytes of keys and values that one position of one request takes, over all groups and planes."""
         elem = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(len(g.spec.keys) * 2 * g.spec.n_kv_heads * g.spec.head_dim * elem for g in self.groups.values())
+        return sum(len(g.spec.keys) * g.spec.n_kv_heads * (g.spec.head_dim + (g.spec.value_dim or g.spec.head_dim)) * elem
+                   for g in self.groups.values())
 
     def free_pages(self) -> Dict[str, int]:
         return {name: g.pool.n_free for name, g in self.groups.items()}

@@ -1,3 +1,4 @@
 from .model_config import (ARCHITECTURES, Architecture, ConfigError, GqaMtpConfig, config_from_dict, load_config,
                            save_config)
 from .registry import Registry
+from .fikevik_config import FikevikConfig

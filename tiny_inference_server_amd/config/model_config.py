@@ -183,7 +183,31 @@ def load_config(model_dir: str):
             raise ConfigError(f"{path}: not valid JSON ({e})") from None
     if not isinstance(raw, dict):
         raise ConfigError(f"{path}: expected a JSON object")
-    return config_from_dict(raw)
+    config = config_from_dict(raw)
+    # an architecture some of whose sizes only the tensors' shapes give completes its configuration from the weight
+    # file's header
+    if hasattr(config, "with_tensor_shapes"):
+        weights = os.path.join(model_dir, "model.safetensors")
+        if os.path.isfile(weights):
+            config = config.with_tensor_shapes(safetensors_shapes(weights))
+    return config
+
+
+def safetensors_shapes(path: str) -> Dict[str, tuple]:
+    """{tensor name: shape} from a safetensors file's header (8 bytes of length, then JSON), without its data."""
+    import struct
+    with open(path, "rb") as f:
+        head = f.read(8)
+        if len(head) != 8:
+            raise ConfigError(f"{path}: too short for a safetensors file")
+        (n,) = struct.unpack("<Q", head)
+        if n > (1 << 30):
+            raise ConfigError(f"{path}: a header of {n} bytes is not a safetensors file's")
+        try:
+            meta = json.loads(f.read(n))
+        except (ValueError, UnicodeDecodeError) as e:
+            raise ConfigError(f"{path}: header is not JSON ({e})") from None
+    return {k: tuple(v["shape"]) for k, v in meta.items() if k != "__metadata__" and isinstance(v, dict) and "shape" in v}
 
 
 def save_config(config, model_dir: str) -> None:

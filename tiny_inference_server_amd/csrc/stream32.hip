@@ -1,0 +1,165 @@
+// Row-wise kernels for models whose residual stream is kept in 32-bit whatever the compute type: scaled embedding,
+// the gated sum followed by an RMS norm (norm after the sum), the closing RMS norm, the per-head norm and output gate
+// of recurrent mixers, and the low-rank decay of gated linear attention.
+//
+// The RMS norm here is x / sqrt(mean(x^2) + eps) * gain, eps under the root. Every sum is taken in 32-bit in an order
+// that depends on the row's width alone. `T` is the compute type (float or bf16): what the next matrix product reads.
+#include "common.h"
+
+TIS_DEFINE_LAST_ERROR(tis_stream32)
+
+static constexpr int S32_THREADS = 256;
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+// x32[r] = table[token[r]] * scale, and the same rows in the compute type
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void embed_scale_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                                                                   float scale, float* __restrict__ out32,
+                                                                   T* __restrict__ outT, int D) {
+  const long r = blockIdx.x;
+  const T* src = table + (long)tokens[r] * D;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    const float v = to_f(src[c]) * scale;
+    out32[r * D + c] = v;
+    if (outT) outT[r * D + c] = from_f<T>(v);
+  }
+}
+
+// r = alpha * x + sigmoid(gate + bias) * (s0 * y0 + s1 * y1);  out = r / sqrt(mean(r^2) + eps) * gain
+// y1 and gate may be null (one branch; no gate).
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void gated_postnorm_kernel(
+    const float* __restrict__ x, const float* __restrict__ y0, long ld0, float s0, const float* __restrict__ y1, long ld1,
+    float s1, const float* __restrict__ gate, long ldg, const float* __restrict__ bias, float alpha,
+    const float* __restrict__ gain, float eps, float* __restrict__ out32, T* __restrict__ outT, int D) {
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    float y = s0 * y0[r * ld0 + c];
+    if (y1) y += s1 * y1[r * ld1 + c];
+    if (gate) y *= sigmoid_f(gate[r * ldg + c] + (bias ? bias[c] : 0.f));
+    const float v = alpha * x[r * D + c] + y;
+    out32[r * D + c] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)D + eps);
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    const float v = out32[r * D + c] * inv * gain[c];
+    out32[r * D + c] = v;
+    if (outT) outT[r * D + c] = from_f<T>(v);
+  }
+}
+
+// out = x / sqrt(mean(x^2) + eps) * gain, from the 32-bit stream into the compute type
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void rmsnorm32_kernel(const float* __restrict__ x, const float* __restrict__ gain,
+                                                                 float eps, T* __restrict__ out, long ldo, int D) {
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    const float v = x[r * D + c];
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)D + eps);
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) out[r * ldo + c] = from_f<T>(x[r * D + c] * inv * gain[c]);
+}
+
+// One wave per (row, head): o / sqrt(mean_over_V(o^2) + eps) * gain * act(g). gain is [V] shared by the heads or
+// [H * V]; act 0: g * sigmoid(g), 1: sigmoid(g).
+template <typename T>
+__global__ __launch_bounds__(TIS_WAVE) void head_norm_gate_kernel(const float* __restrict__ o, long ldo,
+                                                                   const float* __restrict__ g, long ldg,
+                                                                   const float* __restrict__ gain, int gain_per_head,
+                                                                   int act, float eps, T* __restrict__ out, long ldout,
+                                                                   int V) {
+  const long r = blockIdx.x;
+  const int h = blockIdx.y;
+  const float* src = o + r * ldo + (long)h * V;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < V; j += TIS_WAVE) ss += src[j] * src[j];
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / (float)V + eps);
+  for (int j = threadIdx.x; j < V; j += TIS_WAVE) {
+    const float z = g[r * ldg + (long)h * V + j];
+    const float a = act == 0 ? z * sigmoid_f(z) : sigmoid_f(z);
+    out[r * ldout + (long)h * V + j] = from_f<T>(src[j] * inv * gain[gain_per_head ? h * V + j : j] * a);
+  }
+}
+
+// decay[r][c] = sigmoid(z)^(1/tau) with z = sum_k low[r][k] * w2[c][k] + bias[c], as exp(log_sigmoid(z) / tau)
+__global__ __launch_bounds__(S32_THREADS) void lowrank_decay_kernel(const float* __restrict__ low, long ldl, int rank,
+                                                                     const float* __restrict__ w2,
+                                                                     const float* __restrict__ bias, float tau,
+                                                                     float* __restrict__ out, int C) {
+  extern __shared__ float a[];
+  const long r = blockIdx.x;
+  for (int k = threadIdx.x; k < rank; k += S32_THREADS) a[k] = low[r * ldl + k];
+  __syncthreads();
+  for (int c = threadIdx.x; c < C; c += S32_THREADS) {
+    float z = 0.f;
+    const float* w = w2 + (long)c * rank;
+    for (int k = 0; k < rank; ++k) z += a[k] * w[k];
+    z += bias[c];
+    out[r * C + c] = expf(log_sigmoid_f(z) / tau);
+  }
+}
+
+#define S32_DISPATCH(call_f32, call_bf16)                 \
+  if (dtype == TIS_F32) { call_f32; }                     \
+  else if (dtype == TIS_BF16) { call_bf16; }              \
+  else return tis_fail("unknown dtype code %d", dtype);
+
+TIS_EXPORT int tis_embed_scale(int dtype, const void* table, const int* tokens, float scale, float* out32, void* outT,
+                               int rows, int D, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1) return tis_fail("embed_scale: bad size rows=%d width=%d", rows, D);
+  S32_DISPATCH((embed_scale_kernel<float><<<rows, S32_THREADS, 0, stream>>>((const float*)table, tokens, scale, out32, (float*)outT, D)),
+               (embed_scale_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>((const bf16*)table, tokens, scale, out32, (bf16*)outT, D)))
+  return tis_launch_status("embed_scale");
+}
+
+TIS_EXPORT int tis_gated_postnorm(int dtype, const float* x, const float* y0, long ld0, float s0, const float* y1, long ld1,
+                                  float s1, const float* gate, long ldg, const float* bias, float alpha, const float* gain,
+                                  float eps, float* out32, void* outT, int rows, int D, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1 || !x || !y0 || !gain || !out32) return tis_fail("gated_postnorm: bad arguments rows=%d width=%d", rows, D);
+  S32_DISPATCH((gated_postnorm_kernel<float><<<rows, S32_THREADS, 0, stream>>>(x, y0, ld0, s0, y1, ld1, s1, gate, ldg, bias, alpha, gain, eps, out32, (float*)outT, D)),
+               (gated_postnorm_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>(x, y0, ld0, s0, y1, ld1, s1, gate, ldg, bias, alpha, gain, eps, out32, (bf16*)outT, D)))
+  return tis_launch_status("gated_postnorm");
+}
+
+TIS_EXPORT int tis_rmsnorm32(int dtype, const float* x, const float* gain, float eps, void* out, long ldo, int rows, int D,
+                             hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1) return tis_fail("rmsnorm32: bad size rows=%d width=%d", rows, D);
+  S32_DISPATCH((rmsnorm32_kernel<float><<<rows, S32_THREADS, 0, stream>>>(x, gain, eps, (float*)out, ldo, D)),
+               (rmsnorm32_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>(x, gain, eps, (bf16*)out, ldo, D)))
+  return tis_launch_status("rmsnorm32");
+}
+
+TIS_EXPORT int tis_head_norm_gate(int dtype, const float* o, long ldo, const float* g, long ldg, const float* gain,
+                                  int gain_per_head, int act, float eps, void* out, long ldout, int rows, int H, int V,
+                                  hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || H < 1 || H > 65535 || V < 1 || (act != 0 && act != 1))
+    return tis_fail("head_norm_gate: bad size rows=%d heads=%d vdim=%d act=%d", rows, H, V, act);
+  dim3 grid(rows, H);
+  S32_DISPATCH((head_norm_gate_kernel<float><<<grid, TIS_WAVE, 0, stream>>>(o, ldo, g, ldg, gain, gain_per_head, act, eps, (float*)out, ldout, V)),
+               (head_norm_gate_kernel<bf16><<<grid, TIS_WAVE, 0, stream>>>(o, ldo, g, ldg, gain, gain_per_head, act, eps, (bf16*)out, ldout, V)))
+  return tis_launch_status("head_norm_gate");
+}
+
+TIS_EXPORT int tis_lowrank_decay(const float* low, long ldl, int rank, const float* w2, const float* bias, float tau,
+                                 float* out, int rows, int C, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || rank < 1 || rank > 8192 || C < 1 || !(tau > 0.f))
+    return tis_fail("lowrank_decay: bad size rows=%d rank=%d channels=%d tau=%g", rows, rank, C, (double)tau);
+  lowrank_decay_kernel<<<rows, S32_THREADS, rank * sizeof(float), stream>>>(low, ldl, rank, w2, bias, tau, out, C);
+  return tis_launch_status("lowrank_decay");
+}

@@ -57,6 +57,8 @@ class Engine:
             config = load_config(model_dir)
         if config is None:
             raise ValueError("give a model folder or a configuration with tensors")
+        if model_dir is None and tensors is not None and hasattr(config, "with_tensor_shapes"):
+            config = config.with_tensor_shapes({n: tuple(t.shape) for n, t in tensors.items()})
         self.config = config
         arch = ARCHITECTURES.get(config.architecture)
         self.spec = arch.build_spec(config)

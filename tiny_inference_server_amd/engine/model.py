@@ -104,6 +104,7 @@ class Model:
         if isinstance(need, PagedKvNeed):
             ctx.group = cache.group_of[key]
             ctx.plane = cache.groups[ctx.group].plane(key)
+            ctx.page_size = cache.page_size
         elif isinstance(need, StateNeed):
             ctx.state = cache.states[key]
         return ctx

@@ -40,6 +40,9 @@ SOURCES: Dict[str, str] = {
     "gemm_library": "gemm_library.hip",
     "gemm_tiles": "gemm_tiles.hip",
     "sampling": "sampling.hip",
+    "stream32": "stream32.hip",
+    "attention_window": "attention_window.hip",
+    "state_scan": "state_scan.hip",
 }
 HEADERS = ["common.h", "attention_mfma.h"]
 # what a library links beyond the HIP runtime

@@ -101,6 +101,21 @@ _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
                            _I, _I, _I, _I, _P, _P],
 })
 
+_SIGNATURES["stream32"] = ("tis_stream32", {
+    "tis_embed_scale": [_I, _P, _P, _F, _P, _P, _I, _I, _P],
+    "tis_gated_postnorm": [_I, _P, _P, _L, _F, _P, _L, _F, _P, _L, _P, _F, _P, _F, _P, _P, _I, _I, _P],
+    "tis_rmsnorm32": [_I, _P, _P, _F, _P, _L, _I, _I, _P],
+    "tis_head_norm_gate": [_I, _P, _L, _P, _L, _P, _I, _I, _F, _P, _L, _I, _I, _I, _P],
+    "tis_lowrank_decay": [_P, _L, _I, _P, _P, _F, _P, _I, _I, _P],
+})
+_SIGNATURES["attention_window"] = ("tis_attention_window", {
+    "tis_attention_prepare": [_I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P],
+    "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+})
+_SIGNATURES["state_scan"] = ("tis_state_scan", {
+    "tis_state_scan": [_I, _P, _L, _I, _I, _I, _F, _P, _L, _I, _I, _P, _P, _F, _P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _P],
+})
+
 _libs = {}
 
 
@@ -1003,6 +1018,206 @@ class HipOps:
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, head_dim, page_size, int(window),
             float(scale), _ptr(slopes), self._stream())
+        return out
+
+    # ---- a residual stream in 32-bit, norm after the sum ------------------------------------------------
+    # The libraries below are loaded when a model first asks for them: a model that has no such part never
+    # compiles them.
+    def _lazy(self, name):
+        lib = self.__dict__.get("_lib_" + name)
+        if lib is None:
+            lib = self.__dict__["_lib_" + name] = library(name)
+        return lib
+
+    def _f32(self, t, what, n=None):
+        self._check(t, what, torch.float32)
+        if not t.is_contiguous() or (n is not None and t.numel() != n):
+            raise KernelError(f"{what}: expected {n if n is not None else 'some'} contiguous 32-bit floats, got "
+                              f"{tuple(t.shape)}")
+        return t
+
+    def _f32_rows(self, t, what, rows, cols):
+        _rows_view(self._check(t, what, torch.float32), what)
+        if t.shape[0] != rows or t.shape[1] < cols:
+            raise KernelError(f"{what}: {tuple(t.shape)} for {rows} rows of at least {cols}")
+        return t
+
+    def embed_scaled(self, table, tokens, scale: float):
+        """(x32, x): rows of the table times `scale` in 32-bit, and the same rows in the compute type (in a 32-bit
+        engine both are one tensor)."""
+        self._check(table, "embedding table")
+        self._index(tokens, "tokens")
+        n, D = tokens.numel(), table.shape[1]
+        if not table.is_contiguous():
+            raise KernelError("embed_scaled: the table must be contiguous")
+        x32 = torch.empty(n, D, dtype=torch.float32, device=self.device)
+        x = x32 if self.dtype == torch.float32 else self.empty(n, D)
+        self._lazy("stream32").tis_embed_scale(self.code, _ptr(table), _ptr(tokens), float(scale), _ptr(x32),
+                                               _ptr(None if x is x32 else x), n, D, self._stream())
+        return x32, x
+
+    def gated_postnorm(self, x32, branches, gate, gate_bias, alpha: float, gain, eps: float):
+        """norm(alpha * x32 + sigmoid(gate + gate_bias) * sum_i scale_i * y_i) with an RMS norm (eps under the root):
+        (result in 32-bit, result in the compute type). branches: one or two (y [rows, width] 32-bit, scale);
+        gate: [rows, width] 32-bit (a strided view is fine) or None for no gate."""
+        n, D = x32.shape
+        self._f32(x32, "gated_postnorm x", n * D)
+        if not 1 <= len(branches) <= 2:
+            raise KernelError(f"gated_postnorm: {len(branches)} branches (one or two)")
+        for y, _ in branches:
+            self._f32_rows(y, "gated_postnorm branch", n, D)
+        if gate is not None:
+            self._f32_rows(gate, "gated_postnorm gate", n, D)
+            if gate_bias is not None:
+                self._f32(gate_bias, "gated_postnorm gate bias", D)
+        self._f32(gain, "gated_postnorm gain", D)
+        out32 = torch.empty(n, D, dtype=torch.float32, device=self.device)
+        out = out32 if self.dtype == torch.float32 else self.empty(n, D)
+        (y0, s0), (y1, s1) = branches[0], (branches[1] if len(branches) > 1 else (None, 0.0))
+        self._lazy("stream32").tis_gated_postnorm(
+            self.code, _ptr(x32), _ptr(y0), y0.stride(0), float(s0), _ptr(y1), y1.stride(0) if y1 is not None else 0,
+            float(s1), _ptr(gate), gate.stride(0) if gate is not None else 0, _ptr(gate_bias if gate is not None else None),
+            float(alpha), _ptr(gain), float(eps), _ptr(out32), _ptr(None if out is out32 else out), n, D, self._stream())
+        return out32, out
+
+    def rmsnorm32(self, x32, gain, eps: float):
+        """x / sqrt(mean(x^2) + eps) * gain of 32-bit rows, in the compute type."""
+        n, D = x32.shape
+        self._f32(x32, "rmsnorm32 x", n * D)
+        self._f32(gain, "rmsnorm32 gain", D)
+        out = self.empty(n, D)
+        self._lazy("stream32").tis_rmsnorm32(self.code, _ptr(x32), _ptr(gain), float(eps), _ptr(out), out.stride(0), n, D,
+                                             self._stream())
+        return out
+
+    def head_norm_gate(self, o32, gate, gain, n_heads: int, vdim: int, eps: float, act: str):
+        """Per head: o / sqrt(mean(o^2) + eps) * gain * act(gate), in the compute type. o32, gate: [rows, heads*vdim]
+        32-bit (gate may be a strided view); gain: [vdim] shared by the heads or [heads*vdim]; act: "silu" or
+        "sigmoid"."""
+        n = o32.shape[0]
+        W = n_heads * vdim
+        self._f32_rows(o32, "head_norm_gate o", n, W)
+        self._f32_rows(gate, "head_norm_gate gate", n, W)
+        self._check(gain, "head_norm_gate gain", torch.float32)
+        if gain.numel() not in (vdim, W) or not gain.is_contiguous() or act not in ("silu", "sigmoid"):
+            raise KernelError(f"head_norm_gate: gain of {gain.numel()} for {n_heads} heads of {vdim}, act {act!r}")
+        out = self.empty(n, W)
+        self._lazy("stream32").tis_head_norm_gate(
+            self.code, _ptr(o32), o32.stride(0), _ptr(gate), gate.stride(0), _ptr(gain),
+            int(gain.numel() == W and n_heads > 1), 0 if act == "silu" else 1, float(eps), _ptr(out), out.stride(0), n,
+            n_heads, vdim, self._stream())
+        return out
+
+    def lowrank_decay(self, low, w2, bias, tau: float):
+        """sigmoid(low . w2^T + bias)^(1/tau) in 32-bit: low [rows, rank] (a strided view is fine), w2 [channels, rank]."""
+        n, rank = low.shape
+        _rows_view(self._check(low, "lowrank_decay low", torch.float32), "lowrank_decay low")
+        C = w2.shape[0]
+        self._f32(w2, "lowrank_decay w2", C * rank)
+        self._f32(bias, "lowrank_decay bias", C)
+        out = torch.empty(n, C, dtype=torch.float32, device=self.device)
+        self._lazy("stream32").tis_lowrank_decay(_ptr(low), low.stride(0), rank, _ptr(w2), _ptr(bias), float(tau),
+                                                 _ptr(out), n, C, self._stream())
+        return out
+
+    # ---- attention with keys and values of different sizes -----------------------------------------------
+    def _check_kv_plane(self, plane, n_kv_heads, key_dim, value_dim, page_size):
+        self._check(plane, "cache plane")
+        per_page = n_kv_heads * page_size * (key_dim + value_dim)
+        if not plane.is_contiguous() or plane.shape[0] < 1 or plane.numel() != plane.shape[0] * per_page:
+            raise KernelError(f"cache plane {tuple(plane.shape)} does not hold pages of {n_kv_heads} heads x {page_size} "
+                              f"slots x ({key_dim} + {value_dim})")
+
+    def attention_prepare(self, proj, q_off, k_off, v_off, positions, write_slots, plane, n_heads, n_kv_heads, key_dim,
+                          value_dim, page_size, q_gain, k_gain, q_factor, freqs, rot_dims, eps, write_cache=True):
+        """From a row's 32-bit projections (queries at column q_off, keys at k_off, values at v_off): queries
+        [rows, heads*key_dim] in the compute type, normed per head (RMS, gain), rotated in interleaved pairs over the
+        first rot_dims channels (angle = position * freqs[pair]) and multiplied by q_factor[head]; keys normed and
+        rotated alike and values divided by their root mean square go into the pages at write_slots."""
+        n = proj.shape[0]
+        need = max(q_off + n_heads * key_dim, k_off + n_kv_heads * key_dim, v_off + n_kv_heads * value_dim)
+        self._f32_rows(proj, "attention_prepare projections", n, need)
+        self._index(positions, "positions", n)
+        self._f32(q_gain, "query norm gain", key_dim)
+        self._f32(k_gain, "key norm gain", key_dim)
+        self._f32(q_factor, "query factors", n_heads)
+        if rot_dims:
+            self._f32(freqs, "rotary frequencies", rot_dims // 2)
+        if write_cache:
+            self._index(write_slots, "write_slots", n)
+            self._check_kv_plane(plane, n_kv_heads, key_dim, value_dim, page_size)
+        q = self.empty(n, n_heads * key_dim)
+        self._lazy("attention_window").tis_attention_prepare(
+            self.code, _ptr(proj), proj.stride(0), q_off, k_off, v_off, _ptr(positions),
+            _ptr(write_slots if write_cache else None), _ptr(plane if write_cache else None), _ptr(q), q.stride(0),
+            _ptr(q_gain), _ptr(k_gain), _ptr(q_factor), _ptr(freqs if rot_dims else None), int(rot_dims), float(eps), n,
+            n_heads, n_kv_heads, key_dim, value_dim, page_size, self._stream())
+        return q
+
+    def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
+                           scale=None):
+        """Attention of the rows in `batch` over pages whose keys have key_dim and whose values value_dim channels:
+        [rows, heads*value_dim]."""
+        _rows_view(self._check(q, "q"), "q")
+        n = q.shape[0]
+        self._check_kv_plane(plane, n_kv_heads, key_dim, value_dim, page_size)
+        if q.shape[1] != n_heads * key_dim:
+            raise KernelError(f"attention: q width {q.shape[1]} is not heads {n_heads} x key size {key_dim}")
+        tables = batch.block_tables[group]
+        self._check(tables, "block tables", torch.int32)
+        if tables.dim() != 2 or tables.stride(1) != 1:
+            raise KernelError(f"attention: block tables {tuple(tables.shape)} must be 2-d")
+        self._index(batch.positions, "positions", n)
+        self._index(batch.row_seq, "row_seq", n)
+        if batch.max_kv_len > tables.shape[1] * page_size:
+            raise KernelError(f"attention: a row sees {batch.max_kv_len} keys but block tables cover "
+                              f"{tables.shape[1] * page_size}")
+        out = self.empty(n, n_heads * value_dim)
+        self._lazy("attention_window").tis_attention_window(
+            self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
+            _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, key_dim, value_dim, page_size,
+            int(window), float(scale if scale is not None else key_dim ** -0.5), self._stream())
+        return out
+
+    # ---- recurrent mixers with a matrix state per head ---------------------------------------------------
+    @staticmethod
+    def state_scan_floats(kind: str, n_heads: int, dim: int, vdim: int) -> int:
+        """32-bit floats of one request's state: S [heads, dim, vdim]; "gated_max" also keeps its normaliser n [dim]
+        and running maximum per head, once per block of 16 value channels (the kernel's workgroups)."""
+        blocks = -(-vdim // 16)
+        return n_heads * dim * vdim + (n_heads * blocks * (dim + 1) if kind == "gated_max" else 0)
+
+    def state_scan(self, kind, proj, q_off, k_off, v_off, q_scale, state, batch, n_heads, dim, vdim, decay=None,
+                   i_off=0, f_off=0, bias_i=None, bias_f=None, cap=0.0):
+        """Walk the step's rows of every request through its matrix state, in order, and return o [rows, heads*vdim]
+        in 32-bit. kind "decay": S = diag(decay) S + k v^T, o = S^T q. kind "gated_max": scalar log gates per head
+        from the columns i_off, f_off of proj (plus biases, capped by cap * tanh(. / cap)), stabilised by a running
+        maximum, o normalised by max(|n . q|, exp(-m)) + 1e-6. state: [slots, floats] 32-bit, a line per request."""
+        n = proj.shape[0]
+        need = max(q_off + n_heads * dim, k_off + n_heads * dim, v_off + n_heads * vdim)
+        if kind == "gated_max":
+            need = max(need, i_off + n_heads, f_off + n_heads)
+            self._f32(bias_i, "input gate bias", n_heads)
+            self._f32(bias_f, "forget gate bias", n_heads)
+        elif kind == "decay":
+            self._f32_rows(decay, "decays", n, n_heads * dim)
+        else:
+            raise KernelError(f"state_scan: unknown kind {kind!r}")
+        self._f32_rows(proj, "state_scan projections", n, need)
+        self._check(state, "state", torch.float32)
+        if state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < self.state_scan_floats(kind, n_heads, dim, vdim):
+            raise KernelError(f"state_scan: state {tuple(state.shape)} for lines of "
+                              f"{self.state_scan_floats(kind, n_heads, dim, vdim)} floats")
+        self._index(batch.cu_rows, "cu_rows", batch.n_seqs + 1)
+        self._index(batch.seq_slots, "seq_slots", batch.n_seqs)
+        if max(batch.host_slots, default=0) >= state.shape[0]:
+            raise KernelError(f"state_scan: slot {max(batch.host_slots)} of {state.shape[0]}")
+        out = torch.empty(n, n_heads * vdim, dtype=torch.float32, device=self.device)
+        self._lazy("state_scan").tis_state_scan(
+            0 if kind == "decay" else 1, _ptr(proj), proj.stride(0), q_off, k_off, v_off, float(q_scale), _ptr(decay),
+            decay.stride(0) if decay is not None else 0, i_off, f_off, _ptr(bias_i), _ptr(bias_f), float(cap),
+            _ptr(state), state.stride(0), _ptr(batch.cu_rows), _ptr(batch.seq_slots), batch.n_seqs, _ptr(out),
+            out.stride(0), n_heads, dim, vdim, self._stream())
         return out
 
     # ---- sampling ------------------------------------------------------------------------------------

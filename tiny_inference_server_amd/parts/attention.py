@@ -91,3 +91,84 @@ class GqaAttention:
         attn = ops.paged_attention(q, ctx.plane, b, ctx.group, self.n_heads, self.n_kv_heads,
                                    self.head_dim, self.window, self.scale, **extra)
         return ops.linear(attn, self.w_o, residual=residual, reuse_residual=ctx.residual_is_spent)
+
+
+@MIXERS.register("windowed_qknorm_attention")
+class WindowedQkNormAttention:
+    """Grouped-query softmax attention over the last `window` positions (0: all), with keys and values of different
+    sizes. q = x.Wq^T, k = x.Wk^T, v = x.Wv^T; queries and keys are RMS-normed per head (a gain of key_dim entries
+    each, shared by the heads), then the first rot_dims channels of each head are rotated in interleaved pairs
+    (2i, 2i+1) by position * base^(-2i/rot_dims); values are divided by their root mean square and cached so;
+    score = q.k * scale * temp[head]; out = softmax-weighted values of all heads . Wo^T. Norms, angles, scores and
+    the softmax are 32-bit.
+
+    params: width, n_heads, n_kv_heads, key_dim, value_dim, window, rot_dims, rot_base, scale, eps. tensors, stored
+    [out, in]: q (heads*key_dim, width), k (kv_heads*key_dim, width), v (kv_heads*value_dim, width), q_norm, k_norm
+    (key_dim,), temp (heads,), o (width, heads*value_dim).
+    """
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, H, G, kd, vd = (params[k] for k in ("width", "n_heads", "n_kv_heads", "key_dim", "value_dim"))
+        return {"q": (H * kd, w), "k": (G * kd, w), "v": (G * vd, w), "q_norm": (kd,), "k_norm": (kd,), "temp": (H,),
+                "o": (w, H * vd)}
+
+    @classmethod
+    def cache_need(cls, params):
+        return PagedKvNeed(params["n_kv_heads"], params["key_dim"], int(params.get("window", 0)),
+                           value_dim=params["value_dim"])
+
+    def __init__(self, spec, tensors, ops):
+        from .base import to_gain
+        p = spec.params
+        self.ops = ops
+        self.H, self.G, self.kd, self.vd = int(p["n_heads"]), int(p["n_kv_heads"]), int(p["key_dim"]), int(p["value_dim"])
+        if self.H % self.G:
+            raise ValueError(f"{self.H} query heads are not a multiple of {self.G} key/value heads")
+        self.window, self.scale, self.eps = int(p.get("window", 0)), float(p["scale"]), float(p["eps"])
+        self.rot_dims = int(p.get("rot_dims", 0))
+        if self.rot_dims % 2 or self.rot_dims > self.kd:
+            raise ValueError(f"{self.rot_dims} rotated channels of a head of {self.kd}: an even number, at most the head")
+        i = torch.arange(self.rot_dims // 2, dtype=torch.float64)
+        self.freqs = (float(p.get("rot_base", 10000.0)) ** (-2.0 * i / max(1, self.rot_dims))).to(torch.float32).to(ops.device)
+        q, k, v = tensors.of(spec, "q"), tensors.of(spec, "k"), tensors.of(spec, "v")
+        self.input_rows = torch.cat((q, k, v), dim=0)
+        self.k_at, self.v_at = q.shape[0], q.shape[0] + k.shape[0]
+        self._w_in = None
+        self.q_gain, self.k_gain = to_gain(ops, tensors.of(spec, "q_norm")), to_gain(ops, tensors.of(spec, "k_norm"))
+        self.temp = to_gain(ops, tensors.of(spec, "temp"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+        self.same = self.kd == self.vd        # then the pages have the layout every attention kernel reads
+
+    # the matrix-core kernels' work lists, where keys and values are of one size (see GqaAttention)
+    def plan_key(self):
+        if not self.same or not hasattr(self.ops, "plan_attention"):
+            return None
+        return ("attention", self.H, self.G, self.kd, self.window)
+
+    def plan_mode(self, seq_rows):
+        mode = getattr(self.ops, "plan_attention_mode", None)
+        return mode(seq_rows, self.window) if mode is not None and self.same else None
+
+    def plan_rows(self, seq_rows, add, mode=None):
+        return self.ops.plan_attention(self.H, self.G, self.kd, seq_rows, add, mode, self.window)
+
+    def core(self, proj, ctx):
+        ops, b = self.ops, ctx.batch
+        q = ops.attention_prepare(proj, 0, self.k_at, self.v_at, b.positions, b.write_slots[ctx.group], ctx.plane, self.H,
+                                  self.G, self.kd, self.vd, ctx.page_size, self.q_gain, self.k_gain, self.temp,
+                                  self.freqs, self.rot_dims, self.eps, ctx.writes_cache)
+        if self.same:
+            return ops.paged_attention(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, self.window, self.scale)
+        return ops.paged_attention_kv(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, self.vd, ctx.page_size,
+                                      self.window, self.scale)
+
+    def forward_projected(self, proj, ctx):
+        return self.ops.linear(self.core(proj, ctx), self.w_o, out_dtype=torch.float32)
+
+    def forward(self, x, ctx, residual=None):
+        if self._w_in is None:
+            self._w_in = to_compute(self.ops, self.input_rows)
+        proj = self.ops.linear(x, self._w_in, out_dtype=torch.float32)
+        return self.ops.linear(self.core(proj, ctx), self.w_o, residual=residual)

@@ -47,6 +47,7 @@ NORMS: Registry = Registry("norm")
 POSITION_ENCODINGS: Registry = Registry("position encoding")
 ARRANGEMENTS: Registry = Registry("block arrangement")
 STAGE_INPUTS: Registry = Registry("stage input")
+GATES: Registry = Registry("residual gate")
 
 
 @dataclass
@@ -57,7 +58,9 @@ class CallContext:
     each mixer's own context (same batch, that part's cache)."""
     batch: Any                       # engine.batch.StageBatch
     group: Optional[str] = None      # page group of the call's cache, for paged needs
-    plane: Any = None                # [pages, 2, kv heads, page size, head size] for paged needs
+    plane: Any = None                # [pages, 2, kv heads, page size, head size] for paged needs (keys and values of
+                                     # different sizes: [pages, everything a page holds])
+    page_size: int = 0               # slots of a page, for paged needs
     state: Any = None                # [max requests, *shape] for state needs
     writes_cache: bool = True
     residual_is_spent: bool = False  # the caller will not read the residual it passes again: it may be overwritten
@@ -99,7 +102,7 @@ class Tensors:
 
 
 REGISTRIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "position": POSITION_ENCODINGS,
-              "stage_input": STAGE_INPUTS}
+              "stage_input": STAGE_INPUTS, "gate": GATES}
 
 
 def part_class(spec):

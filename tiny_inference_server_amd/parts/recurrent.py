@@ -1,0 +1,121 @@
+"""Recurrent mixers: a matrix state per head and request, kept in 32-bit in the request's state slot."""
+from __future__ import annotations
+
+import torch
+
+from .base import MIXERS, to_compute, to_gain
+from .spec import StateNeed
+
+
+def state_floats(kind: str, n_heads: int, dim: int, vdim: int) -> int:
+    """32-bit floats of one request's state: S [heads, dim, vdim]; kind "gated_max" also keeps its normaliser
+    n [dim] and running maximum per head, once per block of 16 value channels (a workgroup of the scan kernel)."""
+    blocks = -(-vdim // 16)
+    return n_heads * dim * vdim + (n_heads * blocks * (dim + 1) if kind == "gated_max" else 0)
+
+
+class _MatrixStateMixer:
+    """What the two mixers below share: stacked input matrices, the output matrix, the ways in."""
+    graph_safe = True
+
+    def _stack(self, spec, tensors, keys):
+        """The input matrices under `keys`, stacked as stored; returns their first columns in the product."""
+        mats = [tensors.of(spec, k) for k in keys]
+        self.input_rows = torch.cat(mats, dim=0)
+        offs, at = {}, 0
+        for k, m in zip(keys, mats):
+            offs[k] = at
+            at += m.shape[0]
+        self._w_in = None
+        return offs
+
+    def forward_projected(self, proj, ctx):
+        """From this mixer's columns of a 32-bit input product to its result in 32-bit."""
+        return self.ops.linear(self.core(proj, ctx), self.w_o, out_dtype=torch.float32)
+
+    def forward(self, x, ctx, residual=None):
+        if self._w_in is None:
+            self._w_in = to_compute(self.ops, self.input_rows)
+        proj = self.ops.linear(x, self._w_in, out_dtype=torch.float32)
+        return self.ops.linear(self.core(proj, ctx), self.w_o, residual=residual)
+
+
+@MIXERS.register("gated_linear_attention")
+class GatedLinearAttention(_MatrixStateMixer):
+    """Per head S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, with q = x.Wq^T / sqrt(dim), k = x.Wk^T,
+    v = x.Wv^T and a decay per key channel a = sigmoid((x.Wa1^T).Wa2^T + b)^(1/tau). Each head's o is RMS-normed over
+    its value channels (gain of vdim entries, shared by the heads), multiplied by silu(x.Wg^T) and projected by Wo.
+    Decays, state and sums are 32-bit; the state starts at zero.
+
+    params: width, n_heads, dim, vdim, tau, rank, eps. tensors, stored [out, in]: q, k (heads*dim, width), v, g
+    (heads*vdim, width), o (width, heads*vdim), norm (vdim,), a1 (rank, width), a2 (heads*dim, rank), a2_bias.
+    """
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, H, D, V, r = (params[k] for k in ("width", "n_heads", "dim", "vdim", "rank"))
+        return {"q": (H * D, w), "k": (H * D, w), "v": (H * V, w), "g": (H * V, w), "o": (w, H * V), "norm": (V,),
+                "a1": (r, w), "a2": (H * D, r), "a2_bias": (H * D,)}
+
+    @classmethod
+    def cache_need(cls, params):
+        return StateNeed((state_floats("decay", params["n_heads"], params["dim"], params["vdim"]),), "float32")
+
+    def __init__(self, spec, tensors, ops):
+        p = spec.params
+        self.ops = ops
+        self.H, self.D, self.V, self.rank = int(p["n_heads"]), int(p["dim"]), int(p["vdim"]), int(p["rank"])
+        self.tau, self.eps = float(p["tau"]), float(p["eps"])
+        self.at = self._stack(spec, tensors, ("q", "k", "v", "g", "a1"))
+        self.w_a2 = to_gain(ops, tensors.of(spec, "a2"))
+        self.a2_bias = to_gain(ops, tensors.of(spec, "a2_bias"))
+        self.norm_gain = to_gain(ops, tensors.of(spec, "norm"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+
+    def core(self, proj, ctx):
+        ops, at, H, D, V = self.ops, self.at, self.H, self.D, self.V
+        decay = ops.lowrank_decay(proj[:, at["a1"]:at["a1"] + self.rank], self.w_a2, self.a2_bias, self.tau)
+        o = ops.state_scan("decay", proj, at["q"], at["k"], at["v"], D ** -0.5, ctx.state, ctx.batch, H, D, V,
+                           decay=decay)
+        return ops.head_norm_gate(o, proj[:, at["g"]:at["g"] + H * V], self.norm_gain, H, V, self.eps, "silu")
+
+
+@MIXERS.register("matrix_memory")
+class MatrixMemory(_MatrixStateMixer):
+    """A matrix memory with exponential gating. Per head, with log gates i = cap tanh((x.Wi^T + bi) / cap) and
+    f = log sigmoid(cap tanh((x.Wf^T + bf) / cap)) and a running maximum m (which starts at 0):
+    m_t = max(f + m_(t-1), i); S_t = exp(f + m_(t-1) - m_t) S_(t-1) + exp(i - m_t) k v^T; n_t alike with k alone;
+    o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6), q = x.Wq^T / sqrt(dim). Each head's o is divided by its root
+    mean square, the heads side by side are multiplied by a gain and by sigmoid(x.Wg^T), then projected by Wo.
+    Gates, state and sums are 32-bit; S and n start at zero.
+
+    params: width, n_heads, dim, vdim, gate_cap, eps. tensors, stored [out, in]: q, k (heads*dim, width), v, g
+    (heads*vdim, width), o (width, heads*vdim), norm (heads*vdim,), i, f (heads, width), i_bias, f_bias (heads,).
+    """
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, H, D, V = (params[k] for k in ("width", "n_heads", "dim", "vdim"))
+        return {"q": (H * D, w), "k": (H * D, w), "v": (H * V, w), "g": (H * V, w), "o": (w, H * V), "norm": (H * V,),
+                "i": (H, w), "f": (H, w), "i_bias": (H,), "f_bias": (H,)}
+
+    @classmethod
+    def cache_need(cls, params):
+        return StateNeed((state_floats("gated_max", params["n_heads"], params["dim"], params["vdim"]),), "float32")
+
+    def __init__(self, spec, tensors, ops):
+        p = spec.params
+        self.ops = ops
+        self.H, self.D, self.V = int(p["n_heads"]), int(p["dim"]), int(p["vdim"])
+        self.cap, self.eps = float(p["gate_cap"]), float(p["eps"])
+        self.at = self._stack(spec, tensors, ("q", "k", "v", "g", "i", "f"))
+        self.i_bias = to_gain(ops, tensors.of(spec, "i_bias"))
+        self.f_bias = to_gain(ops, tensors.of(spec, "f_bias"))
+        self.norm_gain = to_gain(ops, tensors.of(spec, "norm"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+
+    def core(self, proj, ctx):
+        ops, at, H, D, V = self.ops, self.at, self.H, self.D, self.V
+        o = ops.state_scan("gated_max", proj, at["q"], at["k"], at["v"], D ** -0.5, ctx.state, ctx.batch, H, D, V,
+                           i_off=at["i"], f_off=at["f"], bias_i=self.i_bias, bias_f=self.f_bias, cap=self.cap)
+        return ops.head_norm_gate(o, proj[:, at["g"]:at["g"] + H * V], self.norm_gain, H, V, self.eps, "sigmoid")

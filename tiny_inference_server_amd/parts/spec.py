@@ -34,6 +34,7 @@ class LayerSpec:
     norms in other places; every part whose role is "mixer" gets a cache of its own if its kind asks for one."""
     arrangement: str                      # block arrangement kind, e.g. "prenorm_residual"
     parts: Mapping[str, PartSpec]         # the arrangement's name for the part -> the part
+    params: Mapping[str, Any] = field(default_factory=dict)    # the arrangement's own constants
 
     def part(self, name: str) -> PartSpec:
         try:
@@ -42,7 +43,7 @@ class LayerSpec:
             raise KeyError(f"a {self.arrangement!r} block has no part {name!r}; it has {sorted(self.parts)}") from None
 
     def with_part(self, name: str, spec: PartSpec) -> "LayerSpec":
-        return LayerSpec(self.arrangement, {**self.parts, name: spec})
+        return LayerSpec(self.arrangement, {**self.parts, name: spec}, self.params)
 
     def mixers(self) -> Tuple[Tuple[str, PartSpec], ...]:
         return tuple((n, p) for n, p in self.parts.items() if p.role == "mixer")
@@ -82,10 +83,12 @@ class ModelSpec:
 
 @dataclass(frozen=True)
 class PagedKvNeed:
-    """Keys and values of every position (window 0) or of the last `window` positions."""
+    """Keys and values of every position (window 0) or of the last `window` positions. value_dim: channels of a
+    value where they differ from a key's head_dim (0: the same)."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: int = 0
 
 
 @dataclass(frozen=True)
