@@ -21,7 +21,7 @@ from .engine import Engine
 
 
 def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[str], out: IO[str] = sys.stdout,
-           page_size: int = 16, max_requests: int = 8, heads: bool = False, device: str = "cuda:0",
+           page_size: int = 16, max_requests: int = 4, heads: bool = False, device: str = "cuda:0",
            ops=None) -> int:
     os.makedirs(out_dir, exist_ok=True)
     print(f"[trace_run] loading {model_dir} as {dtype}", file=sys.stderr, flush=True)
@@ -64,7 +64,7 @@ def main(argv: Optional[list] = None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens that live requests hold at any time; the cache pool is made for this many")
     ap.add_argument("--page-size", type=int, default=16)
-    ap.add_argument("--max-requests", type=int, default=8)
+    ap.add_argument("--max-requests", type=int, default=4, help="state slots: the most requests that are live at a time")
     ap.add_argument("--heads", action="store_true", help="also write the prediction heads' logits")
     ap.add_argument("--device", default="cuda:0")
     a = ap.parse_args(argv)
