@@ -145,6 +145,130 @@ class TorchOps:
                 out[r, h * head_dim:(h + 1) * head_dim] = torch.softmax(s, dim=0) @ v[:, h // g]
         return out.to(q.dtype)
 
+    # ---- a residual stream in 32-bit, norm after the sum ---------------------------------------------------
+    def embed_scaled(self, table, tokens, scale):
+        x32 = table[tokens.long()].float() * scale
+        return x32, (x32 if self.dtype == torch.float32 else x32.to(self.dtype))
+
+    def gated_postnorm(self, x32, branches, gate, gate_bias, alpha, gain, eps):
+        y = sum(float(s) * b.float()[:, :x32.shape[1]] for b, s in branches)
+        if gate is not None:
+            y = y * torch.sigmoid(gate.float() + (gate_bias if gate_bias is not None else 0.0))
+        r = alpha * x32 + y
+        out = r / torch.sqrt((r * r).mean(-1, keepdim=True) + eps) * gain
+        return out, (out if self.dtype == torch.float32 else out.to(self.dtype))
+
+    def rmsnorm32(self, x32, gain, eps):
+        return (x32 / torch.sqrt((x32 * x32).mean(-1, keepdim=True) + eps) * gain).to(self.dtype)
+
+    def head_norm_gate(self, o32, gate, gain, n_heads, vdim, eps, act):
+        n = o32.shape[0]
+        o = o32.view(n, n_heads, vdim)
+        o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps)
+        o = o * (gain.view(n_heads, vdim) if gain.numel() == n_heads * vdim else gain)
+        g = gate.float().reshape(n, n_heads, vdim)
+        a = g * torch.sigmoid(g) if act == "silu" else torch.sigmoid(g)
+        return (o * a).reshape(n, n_heads * vdim).to(self.dtype)
+
+    def lowrank_decay(self, low, w2, bias, tau):
+        z = low.float() @ w2.t() + bias
+        return torch.exp(torch.nn.functional.logsigmoid(z) / tau)
+
+    def attention_prepare(self, proj, q_off, k_off, v_off, positions, write_slots, plane, n_heads, n_kv_heads, key_dim,
+                          value_dim, page_size, q_gain, k_gain, q_factor, freqs, rot_dims, eps, write_cache=True):
+        n = proj.shape[0]
+        H, G, kd, vd = n_heads, n_kv_heads, key_dim, value_dim
+
+        def normed(x, gain):
+            return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain
+
+        def turned(x):
+            if not rot_dims:
+                return x
+            ang = positions.float()[:, None] * freqs[None, :]
+            c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+            y = x.clone()
+            y[..., 0:rot_dims:2] = a * c - b * s
+            y[..., 1:rot_dims:2] = b * c + a * s
+            return y
+
+        q = turned(normed(proj[:, q_off:q_off + H * kd].float().reshape(n, H, kd), q_gain)) * q_factor[None, :, None]
+        if write_cache:
+            k = turned(normed(proj[:, k_off:k_off + G * kd].float().reshape(n, G, kd), k_gain)).to(plane.dtype)
+            v = normed(proj[:, v_off:v_off + G * vd].float().reshape(n, G, vd), 1.0).to(plane.dtype)
+            pages = plane.view(plane.shape[0], -1)
+            page, off = write_slots.long() // page_size, write_slots.long() % page_size
+            keys = pages[:, :G * page_size * kd].view(-1, G, page_size, kd)
+            vals = pages[:, G * page_size * kd:].view(-1, G, vd, page_size)
+            keys[page, :, off] = k
+            vals[page, :, :, off] = v
+        return q.reshape(n, H * kd).to(self.dtype)
+
+    def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
+                           scale=None):
+        n = q.shape[0]
+        H, G, kd, vd = n_heads, n_kv_heads, key_dim, value_dim
+        scale = scale if scale is not None else kd ** -0.5
+        tables = batch.block_tables[group]
+        pages = plane.view(plane.shape[0], -1)
+        keys = pages[:, :G * page_size * kd].view(-1, G, page_size, kd)
+        vals = pages[:, G * page_size * kd:].view(-1, G, vd, page_size)
+        out = torch.zeros(n, H * vd, dtype=torch.float32, device=q.device)
+        pos, seq = batch.positions.tolist(), batch.row_seq.tolist()
+        for r in range(n):
+            p = pos[r]
+            js = torch.arange(max(0, p - window + 1) if window > 0 else 0, p + 1)
+            pg = tables[seq[r]].long()[js // page_size]
+            k = keys[pg, :, js % page_size].float()          # [keys, G, kd]
+            v = vals[pg, :, :, js % page_size].float()       # [keys, G, vd]
+            qr = q[r].float().view(H, kd)
+            for h in range(H):
+                w = torch.softmax((k[:, h // (H // G)] @ qr[h]) * scale, dim=0)
+                out[r, h * vd:(h + 1) * vd] = w @ v[:, h // (H // G)]
+        return out.to(q.dtype)
+
+    @staticmethod
+    def state_scan_floats(kind, n_heads, dim, vdim):
+        return n_heads * dim * vdim + (n_heads * -(-vdim // 16) * (dim + 1) if kind == "gated_max" else 0)
+
+    def state_scan(self, kind, proj, q_off, k_off, v_off, q_scale, state, batch, n_heads, dim, vdim, decay=None,
+                   i_off=0, f_off=0, bias_i=None, bias_f=None, cap=0.0):
+        """The same line of state as the kernel keeps (n and m once per block of 16 value channels)."""
+        n, H, D, V = proj.shape[0], n_heads, dim, vdim
+        blocks = -(-V // 16)
+        out = torch.zeros(n, H * V, dtype=torch.float32, device=proj.device)
+        # (the step's device arrays, as the kernel reads them: a kept step's host copies are those of its first run)
+        cu, slots = batch.cu_rows.tolist(), batch.seq_slots.tolist()
+        for k in range(batch.n_seqs):
+            first, rows = cu[k], cu[k + 1] - cu[k]
+            if rows == 0:
+                continue
+            line = state[slots[k]]
+            S = line[:H * D * V].view(H, D, V)
+            nm = line[H * D * V:H * D * V + H * blocks * (D + 1)].view(H, blocks, D + 1) if kind == "gated_max" else None
+            for r in range(first, first + rows):
+                q = proj[r, q_off:q_off + H * D].float().view(H, D) * q_scale
+                kk = proj[r, k_off:k_off + H * D].float().view(H, D)
+                v = proj[r, v_off:v_off + H * V].float().view(H, V)
+                if kind == "decay":
+                    S.copy_(decay[r].view(H, D, 1) * S + kk[:, :, None] * v[:, None, :])
+                    o = torch.einsum("hdv,hd->hv", S, q)
+                else:
+                    gi = cap * torch.tanh((proj[r, i_off:i_off + H].float() + bias_i) / cap)
+                    gf = torch.nn.functional.logsigmoid(cap * torch.tanh((proj[r, f_off:f_off + H].float() + bias_f) / cap))
+                    m = nm[:, 0, D].clone()
+                    m_new = torch.maximum(gf + m, gi)
+                    keep, take = torch.exp(gf + m - m_new), torch.exp(gi - m_new)
+                    S.copy_(keep[:, None, None] * S + take[:, None, None] * kk[:, :, None] * v[:, None, :])
+                    nvec = keep[:, None] * nm[:, 0, :D] + take[:, None] * kk
+                    nm[:, :, :D] = nvec[:, None, :]
+                    nm[:, :, D] = m_new[:, None]
+                    den = torch.maximum((nvec * q).sum(-1).abs(), torch.exp(-m_new)) + 1e-6
+                    o = torch.einsum("hdv,hd->hv", S, q) / den[:, None]
+                out[r] = o.reshape(-1)
+        return out
+
     # ---- sampling ---------------------------------------------------------------------------------------
     def argmax(self, logits):
         return torch.argmax(logits, dim=-1).to(torch.int32)
