@@ -18,6 +18,9 @@ with temperature, top-k, top-p and repetition penalty, finishing, pages given ba
     python bench.py --workload mixed --size 2.1B     64 requests decoding at contexts of 512..8192 while 2,048-token
                                                      portions of further prompts run in the same steps
 
+    python bench.py --workload designs               the Fikevik design beside the grouped-query decoder at equal sizes:
+                                                     prefill and decode throughput of both at a few layer sizes
+
 Each prints one line of the same form; `value` is generated tokens a second over the whole run (serve) or over the
 steps that hold 64 decoding requests and a portion (mixed), `roofline` the sum of the steps' floors (the larger of
 bytes / HBM peak and flops / matrix peak) over the sum of their times.
@@ -281,6 +284,99 @@ def scheduler_workload(a, cfg, layers_full, tensors, heads, page, say, workload=
     return line
 
 
+# Layer sizes for the comparison of designs: (name, width, heads, key/value heads, feed-forward, layers). A head has
+# 128 channels throughout; both designs get the same width, depth, feed-forward and vocabulary.
+DESIGN_SIZES = [("w1024", 1024, 8, 2, 2816, 4), ("w2048", 2048, 16, 4, 5632, 4)]
+
+
+def fikevik_config(width, heads, kv_heads, ff, layers, vocab, window=1024):
+    """Alternating parallel (windowed attention beside a matrix memory) and gated-linear-attention layers."""
+    from tiny_inference_server_amd.config import config_from_dict
+    par = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "mask": {"size": window},
+                              "rot": {"dims": 64, "base": 500000.0}, "scale": 128 ** -0.5},
+                     "right": {"heads": heads // 2, "dim": 128, "vdim": 256, "gate_cap": 15.0},
+                     "left_scale": 1.0, "right_scale": 1.0}}
+    gla = {"type": "gla", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "tau": 16.0, "rank": 16}}
+    return config_from_dict({"architecture": "Fikevik", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+                             "norm": {"eps": 1e-5}, "postln_alpha": 1.0,
+                             "layers": [par if i % 2 == 0 else gla for i in range(layers)]})
+
+
+def design_comparison(a, say):
+    """Prefill (a.prefill_tokens tokens, one prompt) and decode (batch a.batch, context a.context) of the Fikevik design
+    and of the grouped-query decoder without prediction heads at the sizes of DESIGN_SIZES, random weights."""
+    import torch
+
+    from tiny_inference_server_amd.config import GqaMtpConfig
+    from tiny_inference_server_amd.engine import Engine
+    from tiny_inference_server_amd.weights import random_tensors
+    dev, vocab, page = "cuda:0", 32000, 16
+    gen = torch.Generator().manual_seed(a.seed)
+    dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
+    points = {}
+    for name, width, heads, kv_heads, ff, layers in DESIGN_SIZES:
+        designs = {
+            "fikevik": fikevik_config(width, heads, kv_heads, ff, layers, vocab),
+            "gqa": GqaMtpConfig(d_model=width, vocab_size=vocab, max_context=max(8192, a.context), rope_base=500000.0,
+                                n_heads=heads, n_layers=layers, ffn_hidden=ff, group_size=heads // kv_heads, mtp_heads=0,
+                                rms_eps=1e-5, tie_embeddings=False),
+        }
+        for design, cfg in designs.items():
+            say(f"{name} {design}: prefill of {a.prefill_tokens} tokens, decode at batch {a.batch}, context {a.context}")
+            tensors = random_tensors(cfg, a.seed, dtype=a.dtype, device=dev)
+            engine = Engine(config=cfg, tensors=tensors, dtype=a.dtype, page_size=page,
+                            max_tokens=a.batch * (a.context + page) + a.prefill_tokens + page, max_requests=a.batch + 1,
+                            device=dev)
+            ids = torch.randint(0, vocab, (a.prefill_tokens,), generator=gen).tolist()
+            best = None
+            for i in range(4):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                out = engine.step([("prefill", ids, [a.prefill_tokens - 1])])
+                engine.ops.argmax(out.logits).tolist()
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t0
+                engine.close("prefill")
+                if i:
+                    best = dt if best is None else min(best, dt)
+            start_len = a.context - a.steps - a.warmup - 1
+            rids = [f"d{i}" for i in range(a.batch)]
+            for rid in rids:
+                seq = torch.randint(0, vocab, (start_len,), generator=gen).tolist()
+                for p in range(0, start_len, 2048):
+                    engine.step([(rid, seq[p:p + 2048], [])])
+            toks = torch.randint(0, vocab, (a.batch,), generator=gen).tolist()
+            for k in range(a.warmup + a.steps):
+                if k == a.warmup:
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                out = engine.step([(rid, [t], [0]) for rid, t in zip(rids, toks)])
+                toks = engine.ops.argmax(out.logits).tolist()
+            torch.cuda.synchronize()
+            step_s = (time.perf_counter() - t0) / a.steps
+            costs = Costs(engine)
+            points[f"{name}_{design}"] = {
+                "prefill_tok_s": round(a.prefill_tokens / best, 1), "prefill_ms": round(best * 1e3, 3),
+                "decode_tok_s": round(a.batch / step_s, 1), "decode_ms": round(step_s * 1e3, 4),
+                "matrix_elems": costs.matrix_elems + costs.table_elems,
+                "decode_weight_bytes_over_time_frac": round((costs.matrix_elems + costs.table_elems) * costs.elem / step_s / 1e9 / HBM_GBS, 4),
+                "prefill_matrix_flops_frac": round(2.0 * costs.matrix_elems * a.prefill_tokens / best / PEAK_FLOPS[dkey], 4)}
+            del engine, tensors
+            torch.cuda.empty_cache()
+    first = DESIGN_SIZES[0][0]
+    return {"metric": f"decode tok/s at batch {a.batch} of the Fikevik design at {first} ({dkey}); both designs under points",
+            "value": points[f"{first}_fikevik"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
+            "warmup": a.warmup, "ms_per_step": points[f"{first}_fikevik"]["decode_ms"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": dkey,
+            "data": "synthetic: random weights N(0,0.02), uniform random token ids",
+            "config": {"model": "Fikevik beside GqaMtpTransformer", "sizes": [list(s) for s in DESIGN_SIZES],
+                       "global_batch": a.batch, "seq_len": a.context, "prefill_tokens": a.prefill_tokens,
+                       "parallelism": "single-gpu"},
+            "points": points}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -301,7 +397,7 @@ def main() -> int:
     ap.add_argument("--no-trunk-point", dest="trunk_point", action="store_false",
                     help="skip the extra decode measurement without the prediction heads")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--workload", choices=["decode", "serve", "mixed"], default="decode")
+    ap.add_argument("--workload", choices=["decode", "serve", "mixed", "designs"], default="decode")
     ap.add_argument("--requests", type=int, default=64, help="serve, mixed: requests (decoding at once)")
     ap.add_argument("--new-tokens", type=int, default=256, help="serve: tokens generated per request")
     a = ap.parse_args()
@@ -328,6 +424,10 @@ def main() -> int:
 
     # the library's product kernels differ from shape to shape: each new shape is named on stderr before its first launch
     os.environ.setdefault("TIS_TRACE_SHAPES", "1")
+    if a.workload == "designs":
+        torch.cuda.set_device(0)
+        print(json.dumps(design_comparison(a, say)))
+        return 0
 
     from tiny_inference_server_amd.config import ARCHITECTURES
 
