@@ -132,12 +132,17 @@ def test_attention_with_keys_and_values_of_different_sizes(dtype, Hq, G, kd, vd,
         assert torch.isfinite(res[0][1].float()).all()
 
 
+@pytest.mark.parametrize("segment", [64, 8, 5])
 @pytest.mark.parametrize("kind,Hh,D,V", [("decay", 3, 20, 24), ("gated_max", 2, 24, 40), ("decay", 1, 130, 17),
-                                         ("gated_max", 5, 7, 16), ("gated_max", 1, 256, 70)])
-def test_state_scan_against_the_token_by_token_rule(kind, Hh, D, V):
+                                         ("gated_max", 5, 7, 16), ("gated_max", 1, 256, 70), ("gated_max", 2, 64, 130),
+                                         ("decay", 2, 128, 64)])
+def test_state_scan_against_the_token_by_token_rule(kind, Hh, D, V, segment):
     """Portions of three requests in one call, then their next portions and single tokens in further calls, on state
-    lines that start from what an earlier owner left: every result and the final state against plain torch."""
+    lines that start from what an earlier owner left: every result and the final state against plain torch. With
+    segments of 8 and 5 rows the portions of 37, 18 and 40 rows run in segments side by side (beside a request that
+    brings one row), the single tokens after them in order."""
     ops, ref = hip_ops("float32"), TorchOps("cpu", torch.float32)
+    ops.scan_segment = segment
     g = torch.Generator().manual_seed(D)
     floats = ops.state_scan_floats(kind, Hh, D, V)
     assert floats == ref.state_scan_floats(kind, Hh, D, V)

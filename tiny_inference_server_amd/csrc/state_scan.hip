@@ -13,6 +13,17 @@
 // order with nothing else mixed in, so the result of a token does not depend on how a prompt was cut into steps, on the
 // chunk size or on what else is in the batch, bit for bit. State, gates and sums are 32-bit. Kind 1 keeps n and m once
 // per block of value channels (every block needs them, none may read what another has already advanced).
+//
+// Long portions of prompts are cut into segments of `seg_len` tokens that run side by side (`segments` > 0): the same
+// kernel walks every segment from an empty state and leaves the segment's own state, its outputs as if nothing had
+// come before, and what ties them to the past (kind 0: the product of the decays from the segment's start to each
+// token; kind 1: the running maximum, the sum of log forget gates and n . q from the segment's start). A second kernel
+// then walks the segments of a request in order, element by element, to the state at every segment's start and the
+// request's new state; a third adds to every token's output what the state at its segment's start contributes:
+//   kind 0: o_t += (q_t * decay product to t)^T S_start
+//   kind 1: m_t = max(m'_t, F_t + m_start); numerator and n . q are sums of the segment's own part scaled by
+//           exp(m'_t - m_t) and the start's part scaled by exp(F_t + m_start - m_t); o_t as above.
+// Everything is still 32-bit; only the order of additions differs from the token-by-token walk.
 #include "common.h"
 
 TIS_DEFINE_LAST_ERROR(tis_state_scan)
@@ -24,13 +35,26 @@ static constexpr int SC_LDS_BYTES = 60 * 1024;
 
 __device__ __forceinline__ float sc_log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <int KIND, int NS>
+// Workspace of a segmented call, per (request, segment) pair v and head h:
+//   seg_state [v][h][D*V + D + 2]   the segment's own S, n and m (kernel 1); kernel 2 puts the S and n at the segment's
+//                                   start in their place and the m at its start into the last float
+//   cum       [row][H*D]            kind 0: product of the decays from the segment's start to the row
+//   aux       [row][H][3]           kind 1: m', F and n . q of the segment alone
+struct SegArgs {
+  int segments;      // most segments of one request in this call; 0: not segmented
+  int seg_len;
+  float* seg_state;
+  float* cum;
+  float* aux;
+};
+
+template <int KIND, int NS, bool SEG>
 __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
     const float* __restrict__ proj, long ldp, int q_off, int k_off, int v_off, float q_scale,
     const float* __restrict__ decay, long ldd, int i_off, int f_off, const float* __restrict__ bias_i,
     const float* __restrict__ bias_f, float cap, float* __restrict__ state, long state_ld,
     const int* __restrict__ cu_rows, const int* __restrict__ seq_slots, float* __restrict__ out, long ldo, int H, int D,
-    int V, int n_vb, int chunk) {
+    int V, int n_vb, int chunk, SegArgs sg) {
   extern __shared__ float lds[];
   float* sq = lds;                                   // [chunk][D]
   float* sk = sq + chunk * D;                        // [chunk][D]
@@ -38,25 +62,31 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
   float* sv = sa + (KIND == 0 ? chunk * D : chunk * 3);   // [chunk][VB]
   float* part = sv + chunk * SC_VB;                  // [chunk][R][VB + 1]
 
-  const int seq = blockIdx.x, h = blockIdx.y, vb = blockIdx.z, t = threadIdx.x;
-  const int r0 = cu_rows[seq], r1 = cu_rows[seq + 1];
+  const int seq = SEG ? blockIdx.x / sg.segments : blockIdx.x, h = blockIdx.y, vb = blockIdx.z, t = threadIdx.x;
+  int r0 = cu_rows[seq], r1 = cu_rows[seq + 1];
+  if (SEG) {
+    r0 += (blockIdx.x % sg.segments) * sg.seg_len;
+    r1 = min(r1, r0 + sg.seg_len);
+  }
   if (r0 >= r1) return;
-  float* st = state + (long)seq_slots[seq] * state_ld;
-  float* S = st + (long)h * D * V;
-  float* nm = st + (long)H * D * V + ((long)h * n_vb + vb) * (D + 1);     // kind 1: n [D], then m
+  float* st = SEG ? sg.seg_state + ((long)blockIdx.x * H) * ((long)D * V + D + 2) : state + (long)seq_slots[seq] * state_ld;
+  float* S = st + (long)h * (SEG ? (long)D * V + D + 2 : (long)D * V);
+  // kind 1: n [D], then m; once per block of value channels in a request's state line, once per head in a segment's
+  float* nm = SEG ? S + (long)D * V : st + (long)H * D * V + ((long)h * n_vb + vb) * (D + 1);
   const int j = t % SC_VB, s = t / SC_VB;
   const int col = vb * SC_VB + j;
   const bool col_ok = col < V;
 
-  float Sreg[NS], nreg[NS];
-  float m = 0.f;
+  float Sreg[NS], nreg[NS], creg[NS];
+  float m = SEG ? -INFINITY : 0.f, fsum = 0.f;
 #pragma unroll
   for (int e = 0; e < NS; ++e) {
     const int i = s + SC_R * e;
-    Sreg[e] = (i < D && col_ok) ? S[(long)i * V + col] : 0.f;
-    nreg[e] = (KIND == 1 && i < D) ? nm[i] : 0.f;
+    Sreg[e] = (!SEG && i < D && col_ok) ? S[(long)i * V + col] : 0.f;
+    nreg[e] = (!SEG && KIND == 1 && i < D) ? nm[i] : 0.f;
+    creg[e] = 1.f;
   }
-  if (KIND == 1) m = nm[D];
+  if (!SEG && KIND == 1) m = nm[D];
 
   for (int c0 = r0; c0 < r1; c0 += chunk) {
     const int nc = min(chunk, r1 - c0);
@@ -84,9 +114,10 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
       if (KIND == 1) {
         const float gi = sa[c * 3], gf = sa[c * 3 + 1];
         const float m_new = fmaxf(gf + m, gi);
-        keep = expf(gf + m - m_new);
+        keep = expf(gf + m - m_new);      // (an empty segment's m is -inf: nothing is kept of nothing)
         take = expf(gi - m_new);
         m = m_new;
+        fsum += gf;
       }
       const float vj = sv[c * SC_VB + j];
       float acc = 0.f, nq = 0.f;
@@ -97,6 +128,10 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
           const float kk = sk[c * D + i], qq = sq[c * D + i];
           if (KIND == 0) {
             Sreg[e] = sa[c * D + i] * Sreg[e] + kk * vj;
+            if (SEG) {
+              creg[e] *= sa[c * D + i];
+              if (vb == 0 && j == 0) sg.cum[(long)(c0 + c) * H * D + h * D + i] = creg[e];
+            }
           } else {
             Sreg[e] = keep * Sreg[e] + take * (kk * vj);
             nreg[e] = keep * nreg[e] + take * kk;
@@ -109,6 +144,7 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
       if (KIND == 1) {
         if (j == 0) part[(c * SC_R + s) * (SC_VB + 1) + SC_VB] = nq;
         if (t == 0) sa[c * 3 + 2] = m;
+        if (SEG && t == 0 && vb == 0) sg.aux[((long)(c0 + c) * H + h) * 3 + 1] = fsum;
       }
     }
     __syncthreads();
@@ -119,7 +155,11 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
         o += part[(c * SC_R + ss) * (SC_VB + 1) + jj];
         if (KIND == 1) nq += part[(c * SC_R + ss) * (SC_VB + 1) + SC_VB];
       }
-      if (KIND == 1) o /= fmaxf(fabsf(nq), expf(-sa[c * 3 + 2])) + 1e-6f;
+      if (KIND == 1 && !SEG) o /= fmaxf(fabsf(nq), expf(-sa[c * 3 + 2])) + 1e-6f;
+      if (KIND == 1 && SEG && vb == 0 && jj == 0) {
+        sg.aux[((long)(c0 + c) * H + h) * 3] = sa[c * 3 + 2];
+        sg.aux[((long)(c0 + c) * H + h) * 3 + 2] = nq;
+      }
       if (vb * SC_VB + jj < V) out[(long)(c0 + c) * ldo + h * V + vb * SC_VB + jj] = o;
     }
   }
@@ -127,27 +167,165 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
   for (int e = 0; e < NS; ++e) {
     const int i = s + SC_R * e;
     if (i < D && col_ok) S[(long)i * V + col] = Sreg[e];
-    if (KIND == 1 && j == 0 && i < D) nm[i] = nreg[e];
+    if (KIND == 1 && j == 0 && i < D && (!SEG || vb == 0)) nm[i] = nreg[e];
   }
-  if (KIND == 1 && t == 0) nm[D] = m;
+  if (KIND == 1 && t == 0 && (!SEG || vb == 0)) nm[D] = m;
+}
+
+// Kernel 2 of a segmented call: one thread per element of a head's S (and of n), segment after segment in order. What
+// the first kernel left as a segment's own state is replaced by the state at the segment's start; the request's state
+// line receives the state after its last row.
+template <int KIND>
+__global__ __launch_bounds__(SC_THREADS) void segment_states_kernel(float* __restrict__ state, long state_ld,
+                                                                    const int* __restrict__ cu_rows,
+                                                                    const int* __restrict__ seq_slots, int H, int D,
+                                                                    int V, int n_vb, SegArgs sg) {
+  const int seq = blockIdx.x, h = blockIdx.y;
+  const int r0 = cu_rows[seq], r1 = cu_rows[seq + 1];
+  if (r0 >= r1) return;
+  const int el = blockIdx.z * SC_THREADS + threadIdx.x;      // [0, D*V): S; [D*V, D*V + D): n
+  if (el >= D * V + (KIND == 1 ? D : 0)) return;
+  const bool is_n = el >= D * V;
+  const int i = is_n ? el - D * V : el / V;
+  float* st = state + (long)seq_slots[seq] * state_ld;
+  const long per = (long)D * V + D + 2;
+  float x = is_n ? st[(long)H * D * V + (long)h * n_vb * (D + 1) + i] : st[(long)h * D * V + el];
+  float m = KIND == 1 ? st[(long)H * D * V + (long)h * n_vb * (D + 1) + D] : 0.f;
+  const int n_seg = (r1 - r0 + sg.seg_len - 1) / sg.seg_len;
+  for (int g = 0; g < n_seg; ++g) {
+    float* own = sg.seg_state + (((long)seq * sg.segments + g) * H + h) * per;
+    const int last = min(r1, r0 + (g + 1) * sg.seg_len) - 1;
+    const float mine = own[el];
+    float next, m_next = 0.f;
+    if (KIND == 0) {
+      next = sg.cum[(long)last * H * D + h * D + i] * x + mine;
+    } else {
+      const float m_own = own[per - 2], f_all = sg.aux[((long)last * H + h) * 3 + 1];
+      m_next = fmaxf(f_all + m, m_own);
+      next = expf(f_all + m - m_next) * x + expf(m_own - m_next) * mine;
+    }
+    own[el] = x;
+    if (KIND == 1 && el == 0) own[per - 1] = m;
+    x = next;
+    m = m_next;
+  }
+  if (is_n) {
+    for (int b = 0; b < n_vb; ++b) st[(long)H * D * V + ((long)h * n_vb + b) * (D + 1) + i] = x;
+  } else {
+    st[(long)h * D * V + el] = x;
+  }
+  if (KIND == 1 && el == 0)
+    for (int b = 0; b < n_vb; ++b) st[(long)H * D * V + ((long)h * n_vb + b) * (D + 1) + D] = m;
+}
+
+// Kernel 3 of a segmented call: what the state at a segment's start adds to its rows. One workgroup per (request and
+// segment, head, 64 value channels); rows in tiles of 32, a thread owns one channel for 8 rows.
+static constexpr int SG_COLS = 64, SG_ROWS = 32;
+
+template <int KIND>
+__global__ __launch_bounds__(SC_THREADS) void segment_outputs_kernel(const float* __restrict__ proj, long ldp, int q_off,
+                                                                     float q_scale, const int* __restrict__ cu_rows,
+                                                                     float* __restrict__ out, long ldo, int H, int D,
+                                                                     int V, SegArgs sg) {
+  extern __shared__ float lds[];
+  float* s0 = lds;                       // [D][SG_COLS]
+  float* qt = s0 + D * SG_COLS;          // [SG_ROWS][D + 1]
+  float* qn = qt + SG_ROWS * (D + 1);    // [SG_ROWS] kind 1: q . n_start
+  const int seq = blockIdx.x / sg.segments, g = blockIdx.x % sg.segments, h = blockIdx.y, t = threadIdx.x;
+  const int r0 = cu_rows[seq] + g * sg.seg_len, r1 = min(cu_rows[seq + 1], r0 + sg.seg_len);
+  if (r0 >= r1) return;
+  const long per = (long)D * V + D + 2;
+  const float* start = sg.seg_state + ((long)blockIdx.x * H + h) * per;
+  const int c0 = blockIdx.z * SG_COLS, col = t % SG_COLS, rg = t / SG_COLS;      // rg: 0..3, rows rg*8 .. rg*8+7
+  for (int idx = t; idx < D * SG_COLS; idx += SC_THREADS) {
+    const int i = idx / SG_COLS, cc = idx - i * SG_COLS;
+    s0[idx] = c0 + cc < V ? start[(long)i * V + c0 + cc] : 0.f;
+  }
+  const float m0 = KIND == 1 ? start[per - 1] : 0.f;
+  for (int t0 = r0; t0 < r1; t0 += SG_ROWS) {
+    const int nr = min(SG_ROWS, r1 - t0);
+    __syncthreads();
+    for (int idx = t; idx < nr * D; idx += SC_THREADS) {
+      const int r = idx / D, i = idx - r * D;
+      float q = proj[(long)(t0 + r) * ldp + q_off + h * D + i] * q_scale;
+      if (KIND == 0) q *= sg.cum[(long)(t0 + r) * H * D + h * D + i];
+      qt[r * (D + 1) + i] = q;
+    }
+    __syncthreads();
+    if (KIND == 1 && t < nr) {
+      float a = 0.f;
+      for (int i = 0; i < D; ++i) a += qt[t * (D + 1) + i] * start[(long)D * V + i];
+      qn[t] = a;
+    }
+    float acc[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = 0.f;
+    for (int i = 0; i < D; ++i) {
+      const float sv = s0[i * SG_COLS + col];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc[k] += qt[(rg * 8 + k) * (D + 1) + i] * sv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int r = rg * 8 + k;
+      if (r < nr && c0 + col < V) {
+        float* o = out + (long)(t0 + r) * ldo + h * V + c0 + col;
+        if (KIND == 0) {
+          *o += acc[k];
+        } else {
+          const float* a = sg.aux + ((long)(t0 + r) * H + h) * 3;
+          const float m_own = a[0], m_t = fmaxf(m_own, a[1] + m0);
+          const float w_own = expf(m_own - m_t), w_start = expf(a[1] + m0 - m_t);
+          const float nq = w_own * a[2] + w_start * qn[r];
+          *o = (w_own * *o + w_start * acc[k]) / (fmaxf(fabsf(nq), expf(-m_t)) + 1e-6f);
+        }
+      }
+    }
+  }
 }
 
 template <int KIND>
 static int launch_scan(int ns, dim3 grid, size_t lds, hipStream_t stream, const float* proj, long ldp, int q_off, int k_off,
                        int v_off, float q_scale, const float* decay, long ldd, int i_off, int f_off, const float* bias_i,
                        const float* bias_f, float cap, float* state, long state_ld, const int* cu_rows,
-                       const int* seq_slots, float* out, long ldo, int H, int D, int V, int n_vb, int chunk) {
+                       const int* seq_slots, float* out, long ldo, int H, int D, int V, int n_vb, int chunk, SegArgs sg) {
 #define SC_LAUNCH(NS)                                                                                                   \
-  state_scan_kernel<KIND, NS><<<grid, SC_THREADS, lds, stream>>>(proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd,   \
-                                                                 i_off, f_off, bias_i, bias_f, cap, state, state_ld,    \
-                                                                 cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk)
-  if (ns <= 1) SC_LAUNCH(1);
-  else if (ns <= 2) SC_LAUNCH(2);
-  else if (ns <= 4) SC_LAUNCH(4);
-  else if (ns <= 8) SC_LAUNCH(8);
-  else SC_LAUNCH(16);
+  if (sg.segments)                                                                                                      \
+    state_scan_kernel<KIND, NS, true><<<grid, SC_THREADS, lds, stream>>>(                                               \
+        proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off, bias_i, bias_f, cap, state, state_ld,        \
+        cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);                                                        \
+  else                                                                                                                  \
+    state_scan_kernel<KIND, NS, false><<<grid, SC_THREADS, lds, stream>>>(                                              \
+        proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off, bias_i, bias_f, cap, state, state_ld,        \
+        cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg)
+  if (ns <= 1) { SC_LAUNCH(1); }
+  else if (ns <= 2) { SC_LAUNCH(2); }
+  else if (ns <= 4) { SC_LAUNCH(4); }
+  else if (ns <= 8) { SC_LAUNCH(8); }
+  else { SC_LAUNCH(16); }
 #undef SC_LAUNCH
-  return tis_launch_status("state_scan");
+  if (tis_launch_status("state_scan")) return -1;
+  if (!sg.segments) return 0;
+  const int n_seqs = grid.x / sg.segments;
+  const int elems = D * V + (KIND == 1 ? D : 0);
+  segment_states_kernel<KIND><<<dim3(n_seqs, H, (elems + SC_THREADS - 1) / SC_THREADS), SC_THREADS, 0, stream>>>(
+      state, state_ld, cu_rows, seq_slots, H, D, V, n_vb, sg);
+  if (tis_launch_status("segment_states")) return -1;
+  const size_t lds3 = sizeof(float) * ((size_t)D * SG_COLS + (size_t)SG_ROWS * (D + 1) + SG_ROWS);
+  segment_outputs_kernel<KIND><<<dim3(grid.x, H, (V + SG_COLS - 1) / SG_COLS), SC_THREADS, lds3, stream>>>(
+      proj, ldp, q_off, q_scale, cu_rows, out, ldo, H, D, V, sg);
+  return tis_launch_status("segment_outputs");
+}
+
+// Whether heads of D key channels can be run in segments (the third kernel keeps 64 columns of a state in LDS).
+TIS_EXPORT int tis_state_scan_segmentable(int D) {
+  return sizeof(float) * ((size_t)D * SG_COLS + (size_t)SG_ROWS * (D + 1) + SG_ROWS) <= 64 * 1024;
+}
+
+// 32-bit floats of the workspace a segmented call needs: the states, then `rows` lines of decay products or gate sums.
+TIS_EXPORT long tis_state_scan_workspace(int kind, int n_seqs, int segments, int rows, int H, int D, int V) {
+  return (long)n_seqs * segments * H * ((long)D * V + D + 2) + (kind == 0 ? (long)rows * H * D : (long)rows * H * 3);
 }
 
 // Floats of one request's state: S for every head, and for kind 1 also n and m per head and block of value channels.
@@ -160,7 +338,7 @@ TIS_EXPORT int tis_state_scan(int kind, const float* proj, long ldp, int q_off, 
                               const float* decay, long ldd, int i_off, int f_off, const float* bias_i,
                               const float* bias_f, float cap, float* state, long state_ld, const int* cu_rows,
                               const int* seq_slots, int n_seqs, float* out, long ldo, int H, int D, int V,
-                              hipStream_t stream) {
+                              int segments, int seg_len, int rows, float* workspace, hipStream_t stream) {
   if (n_seqs == 0) return 0;
   if (n_seqs < 0 || H < 1 || H > 65535 || D < 1 || D > SC_R * 16 || V < 1)
     return tis_fail("state_scan: bad size requests=%d heads=%d key channels=%d (at most %d) value channels=%d", n_seqs, H,
@@ -179,11 +357,24 @@ TIS_EXPORT int tis_state_scan(int kind, const float* proj, long ldp, int q_off, 
   };
   while (chunk > 1 && bytes(chunk) > SC_LDS_BYTES) chunk /= 2;
   if (bytes(chunk) > SC_LDS_BYTES) return tis_fail("state_scan: %d key channels do not fit the chunk buffers", D);
-  dim3 grid(n_seqs, H, n_vb);
+  SegArgs sg = {0, 0, nullptr, nullptr, nullptr};
+  if (segments > 0) {
+    if (seg_len < 1 || rows < 1 || !workspace || (long)n_seqs * segments > 0x7fffffffL)
+      return tis_fail("state_scan: %d segments of %d rows need a workspace", segments, seg_len);
+    sg.segments = segments;
+    sg.seg_len = seg_len;
+    sg.seg_state = workspace;
+    float* lines = workspace + (long)n_seqs * segments * H * ((long)D * V + D + 2);
+    sg.cum = kind == 0 ? lines : nullptr;
+    sg.aux = kind == 1 ? lines : nullptr;
+    if (sizeof(float) * ((size_t)D * SG_COLS + (size_t)SG_ROWS * (D + 1) + SG_ROWS) > 64 * 1024)
+      return tis_fail("state_scan: %d key channels do not fit the segment kernels (see tis_state_scan_segmentable)", D);
+  }
+  dim3 grid(segments > 0 ? n_seqs * segments : n_seqs, H, n_vb);
   const int ns = (D + SC_R - 1) / SC_R;
   if (kind == 0)
     return launch_scan<0>(ns, grid, bytes(chunk), stream, proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off,
-                          bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk);
+                          bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);
   return launch_scan<1>(ns, grid, bytes(chunk), stream, proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off,
-                        bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk);
+                        bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);
 }

@@ -113,7 +113,8 @@ _SIGNATURES["attention_window"] = ("tis_attention_window", {
     "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _P],
 })
 _SIGNATURES["state_scan"] = ("tis_state_scan", {
-    "tis_state_scan": [_I, _P, _L, _I, _I, _I, _F, _P, _L, _I, _I, _P, _P, _F, _P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _P],
+    "tis_state_scan": [_I, _P, _L, _I, _I, _I, _F, _P, _L, _I, _I, _P, _P, _F, _P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _I,
+                       _I, _I, _P, _P],
 })
 
 _libs = {}
@@ -1192,7 +1193,11 @@ class HipOps:
         """Walk the step's rows of every request through its matrix state, in order, and return o [rows, heads*vdim]
         in 32-bit. kind "decay": S = diag(decay) S + k v^T, o = S^T q. kind "gated_max": scalar log gates per head
         from the columns i_off, f_off of proj (plus biases, capped by cap * tanh(. / cap)), stabilised by a running
-        maximum, o normalised by max(|n . q|, exp(-m)) + 1e-6. state: [slots, floats] 32-bit, a line per request."""
+        maximum, o normalised by max(|n . q|, exp(-m)) + 1e-6. state: [slots, floats] 32-bit, a line per request.
+
+        A step whose longest portion has at least two segments' rows (self.scan_segment, 64) is run in segments side
+        by side, with a second pass for the states at the segments' starts and a third for what they add to the
+        rows' outputs; shorter portions and single tokens are walked in order by one kernel."""
         n = proj.shape[0]
         need = max(q_off + n_heads * dim, k_off + n_heads * dim, v_off + n_heads * vdim)
         if kind == "gated_max":
@@ -1213,11 +1218,20 @@ class HipOps:
         if max(batch.host_slots, default=0) >= state.shape[0]:
             raise KernelError(f"state_scan: slot {max(batch.host_slots)} of {state.shape[0]}")
         out = torch.empty(n, n_heads * vdim, dtype=torch.float32, device=self.device)
-        self._lazy("state_scan").tis_state_scan(
+        lib = self._lazy("state_scan")
+        seg_len = int(getattr(self, "scan_segment", 64))
+        segments, workspace = 0, None
+        if seg_len > 0 and batch.max_seq_rows >= 2 * seg_len and lib.cdll.tis_state_scan_segmentable(dim):
+            segments = -(-batch.max_seq_rows // seg_len)
+            lib.cdll.tis_state_scan_workspace.restype = c_long
+            floats = lib.cdll.tis_state_scan_workspace(0 if kind == "decay" else 1, batch.n_seqs, segments, n, n_heads,
+                                                       dim, vdim)
+            workspace = torch.empty(floats, dtype=torch.float32, device=self.device)
+        lib.tis_state_scan(
             0 if kind == "decay" else 1, _ptr(proj), proj.stride(0), q_off, k_off, v_off, float(q_scale), _ptr(decay),
             decay.stride(0) if decay is not None else 0, i_off, f_off, _ptr(bias_i), _ptr(bias_f), float(cap),
             _ptr(state), state.stride(0), _ptr(batch.cu_rows), _ptr(batch.seq_slots), batch.n_seqs, _ptr(out),
-            out.stride(0), n_heads, dim, vdim, self._stream())
+            out.stride(0), n_heads, dim, vdim, segments, seg_len, n, _ptr(workspace), self._stream())
         return out
 
     # ---- sampling ------------------------------------------------------------------------------------
