@@ -7,7 +7,8 @@
 //           with i = cap tanh((x_i + b_i) / cap), f = log sigmoid(cap tanh((x_f + b_f) / cap)).
 //
 // One workgroup per (request of the step, head, block of 16 value channels). Thread (s, j) owns the state's column j
-// for the key channels s, s + 16, s + 32, ... in registers, from the request's state slot before the first token to
+// for the NS key channels from s * NS on in registers (a token's q, k and decays lie in LDS rows of 16 * NS floats,
+// zeros beyond the head's channels, so a thread reads its share in 16-byte pieces), from the request's state slot before the first token to
 // the slot after the last. Tokens are taken in chunks: a chunk's q, k, v and gates go into LDS, the 16 threads of a
 // column leave a partial o per token there, and one pass adds them up. Each state element sees its tokens strictly in
 // order with nothing else mixed in, so the result of a token does not depend on how a prompt was cut into steps, on the
@@ -55,11 +56,12 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
     const float* __restrict__ bias_f, float cap, float* __restrict__ state, long state_ld,
     const int* __restrict__ cu_rows, const int* __restrict__ seq_slots, float* __restrict__ out, long ldo, int H, int D,
     int V, int n_vb, int chunk, SegArgs sg) {
-  extern __shared__ float lds[];
-  float* sq = lds;                                   // [chunk][D]
-  float* sk = sq + chunk * D;                        // [chunk][D]
-  float* sa = sk + chunk * D;                        // kind 0: [chunk][D] decays; kind 1: [chunk][3] gates i, f and m
-  float* sv = sa + (KIND == 0 ? chunk * D : chunk * 3);   // [chunk][VB]
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  constexpr int DP = SC_R * NS;                      // a token's row in LDS: the head's channels, then zeros
+  float* sq = lds;                                   // [chunk][DP]
+  float* sk = sq + chunk * DP;                       // [chunk][DP]
+  float* sa = sk + chunk * DP;                       // kind 0: [chunk][DP] decays; kind 1: [chunk][4] gates i, f and m
+  float* sv = sa + (KIND == 0 ? chunk * DP : chunk * 4);  // [chunk][VB]
   float* part = sv + chunk * SC_VB;                  // [chunk][R][VB + 1]
 
   const int seq = SEG ? blockIdx.x / sg.segments : blockIdx.x, h = blockIdx.y, vb = blockIdx.z, t = threadIdx.x;
@@ -81,7 +83,7 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
   float m = SEG ? -INFINITY : 0.f, fsum = 0.f;
 #pragma unroll
   for (int e = 0; e < NS; ++e) {
-    const int i = s + SC_R * e;
+    const int i = s * NS + e;
     Sreg[e] = (!SEG && i < D && col_ok) ? S[(long)i * V + col] : 0.f;
     nreg[e] = (!SEG && KIND == 1 && i < D) ? nm[i] : 0.f;
     creg[e] = 1.f;
@@ -91,12 +93,13 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
   for (int c0 = r0; c0 < r1; c0 += chunk) {
     const int nc = min(chunk, r1 - c0);
     __syncthreads();
-    for (int idx = t; idx < nc * D; idx += SC_THREADS) {
-      const int c = idx / D, i = idx - c * D;
+    for (int idx = t; idx < nc * DP; idx += SC_THREADS) {
+      const int c = idx / DP, i = idx - c * DP;
       const float* row = proj + (long)(c0 + c) * ldp;
-      sq[idx] = row[q_off + h * D + i] * q_scale;
-      sk[idx] = row[k_off + h * D + i];
-      if (KIND == 0) sa[idx] = decay[(long)(c0 + c) * ldd + h * D + i];
+      const bool in = i < D;
+      sq[idx] = in ? row[q_off + h * D + i] * q_scale : 0.f;
+      sk[idx] = in ? row[k_off + h * D + i] : 0.f;
+      if (KIND == 0) sa[idx] = in ? decay[(long)(c0 + c) * ldd + h * D + i] : 0.f;
     }
     for (int idx = t; idx < nc * SC_VB; idx += SC_THREADS) {
       const int c = idx / SC_VB, jj = idx - c * SC_VB;
@@ -105,14 +108,14 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
     if (KIND == 1 && t < nc) {
       const float* row = proj + (long)(c0 + t) * ldp;
       const float xi = row[i_off + h] + bias_i[h], xf = row[f_off + h] + bias_f[h];
-      sa[t * 3] = cap * tanhf(xi / cap);
-      sa[t * 3 + 1] = sc_log_sigmoid(cap * tanhf(xf / cap));
+      sa[t * 4] = cap * tanhf(xi / cap);
+      sa[t * 4 + 1] = sc_log_sigmoid(cap * tanhf(xf / cap));
     }
     __syncthreads();
     for (int c = 0; c < nc; ++c) {
       float keep = 1.f, take = 1.f;
       if (KIND == 1) {
-        const float gi = sa[c * 3], gf = sa[c * 3 + 1];
+        const float gi = sa[c * 4], gf = sa[c * 4 + 1];
         const float m_new = fmaxf(gf + m, gi);
         keep = expf(gf + m - m_new);      // (an empty segment's m is -inf: nothing is kept of nothing)
         take = expf(gi - m_new);
@@ -121,29 +124,45 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
       }
       const float vj = sv[c * SC_VB + j];
       float acc = 0.f, nq = 0.f;
+      float kk[NS], qq[NS], aa[NS];
+      const int at = c * DP + s * NS;
+      if (NS % 4 == 0) {
+#pragma unroll
+        for (int e = 0; e < NS; e += 4) {
+          *reinterpret_cast<float4*>(kk + e) = *reinterpret_cast<const float4*>(sk + at + e);
+          *reinterpret_cast<float4*>(qq + e) = *reinterpret_cast<const float4*>(sq + at + e);
+          if (KIND == 0) *reinterpret_cast<float4*>(aa + e) = *reinterpret_cast<const float4*>(sa + at + e);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < NS; ++e) {
+          kk[e] = sk[at + e];
+          qq[e] = sq[at + e];
+          if (KIND == 0) aa[e] = sa[at + e];
+        }
+      }
+      // (channels beyond the head's are zeros in k and q: their state stays zero and adds nothing)
 #pragma unroll
       for (int e = 0; e < NS; ++e) {
-        const int i = s + SC_R * e;
-        if (i < D) {
-          const float kk = sk[c * D + i], qq = sq[c * D + i];
-          if (KIND == 0) {
-            Sreg[e] = sa[c * D + i] * Sreg[e] + kk * vj;
-            if (SEG) {
-              creg[e] *= sa[c * D + i];
-              if (vb == 0 && j == 0) sg.cum[(long)(c0 + c) * H * D + h * D + i] = creg[e];
-            }
-          } else {
-            Sreg[e] = keep * Sreg[e] + take * (kk * vj);
-            nreg[e] = keep * nreg[e] + take * kk;
-            nq += nreg[e] * qq;
-          }
-          acc += Sreg[e] * qq;
+        if (KIND == 0) {
+          Sreg[e] = aa[e] * Sreg[e] + kk[e] * vj;
+          if (SEG) creg[e] *= aa[e];
+        } else {
+          Sreg[e] = keep * Sreg[e] + take * (kk[e] * vj);
+          nreg[e] = keep * nreg[e] + take * kk[e];
+          nq += nreg[e] * qq[e];
         }
+        acc += Sreg[e] * qq[e];
+      }
+      if (KIND == 0 && SEG && vb == 0 && j == 0) {
+#pragma unroll
+        for (int e = 0; e < NS; ++e)
+          if (s * NS + e < D) sg.cum[(long)(c0 + c) * H * D + h * D + s * NS + e] = creg[e];
       }
       part[(c * SC_R + s) * (SC_VB + 1) + j] = acc;
       if (KIND == 1) {
         if (j == 0) part[(c * SC_R + s) * (SC_VB + 1) + SC_VB] = nq;
-        if (t == 0) sa[c * 3 + 2] = m;
+        if (t == 0) sa[c * 4 + 2] = m;
         if (SEG && t == 0 && vb == 0) sg.aux[((long)(c0 + c) * H + h) * 3 + 1] = fsum;
       }
     }
@@ -155,9 +174,9 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
         o += part[(c * SC_R + ss) * (SC_VB + 1) + jj];
         if (KIND == 1) nq += part[(c * SC_R + ss) * (SC_VB + 1) + SC_VB];
       }
-      if (KIND == 1 && !SEG) o /= fmaxf(fabsf(nq), expf(-sa[c * 3 + 2])) + 1e-6f;
+      if (KIND == 1 && !SEG) o /= fmaxf(fabsf(nq), expf(-sa[c * 4 + 2])) + 1e-6f;
       if (KIND == 1 && SEG && vb == 0 && jj == 0) {
-        sg.aux[((long)(c0 + c) * H + h) * 3] = sa[c * 3 + 2];
+        sg.aux[((long)(c0 + c) * H + h) * 3] = sa[c * 4 + 2];
         sg.aux[((long)(c0 + c) * H + h) * 3 + 2] = nq;
       }
       if (vb * SC_VB + jj < V) out[(long)(c0 + c) * ldo + h * V + vb * SC_VB + jj] = o;
@@ -165,7 +184,7 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
   }
 #pragma unroll
   for (int e = 0; e < NS; ++e) {
-    const int i = s + SC_R * e;
+    const int i = s * NS + e;
     if (i < D && col_ok) S[(long)i * V + col] = Sreg[e];
     if (KIND == 1 && j == 0 && i < D && (!SEG || vb == 0)) nm[i] = nreg[e];
   }
@@ -227,7 +246,7 @@ __global__ __launch_bounds__(SC_THREADS) void segment_outputs_kernel(const float
                                                                      float q_scale, const int* __restrict__ cu_rows,
                                                                      float* __restrict__ out, long ldo, int H, int D,
                                                                      int V, SegArgs sg) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* s0 = lds;                       // [D][SG_COLS]
   float* qt = s0 + D * SG_COLS;          // [SG_ROWS][D + 1]
   float* qn = qt + SG_ROWS * (D + 1);    // [SG_ROWS] kind 1: q . n_start
@@ -236,7 +255,7 @@ __global__ __launch_bounds__(SC_THREADS) void segment_outputs_kernel(const float
   if (r0 >= r1) return;
   const long per = (long)D * V + D + 2;
   const float* start = sg.seg_state + ((long)blockIdx.x * H + h) * per;
-  const int c0 = blockIdx.z * SG_COLS, col = t % SG_COLS, rg = t / SG_COLS;      // rg: 0..3, rows rg*8 .. rg*8+7
+  const int c0 = blockIdx.z * SG_COLS, cg = t % 16, rg = t / 16;      // columns cg*4 .. cg*4+3, rows rg*2, rg*2+1
   for (int idx = t; idx < D * SG_COLS; idx += SC_THREADS) {
     const int i = idx / SG_COLS, cc = idx - i * SG_COLS;
     s0[idx] = c0 + cc < V ? start[(long)i * V + c0 + cc] : 0.f;
@@ -261,14 +280,15 @@ __global__ __launch_bounds__(SC_THREADS) void segment_outputs_kernel(const float
 #pragma unroll
     for (int k = 0; k < 8; ++k) acc[k] = 0.f;
     for (int i = 0; i < D; ++i) {
-      const float sv = s0[i * SG_COLS + col];
-#pragma unroll
-      for (int k = 0; k < 8; ++k) acc[k] += qt[(rg * 8 + k) * (D + 1) + i] * sv;
+      const float4 sv = *reinterpret_cast<const float4*>(s0 + i * SG_COLS + cg * 4);
+      const float qa = qt[(rg * 2) * (D + 1) + i], qb = qt[(rg * 2 + 1) * (D + 1) + i];
+      acc[0] += qa * sv.x; acc[1] += qa * sv.y; acc[2] += qa * sv.z; acc[3] += qa * sv.w;
+      acc[4] += qb * sv.x; acc[5] += qb * sv.y; acc[6] += qb * sv.z; acc[7] += qb * sv.w;
     }
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-      const int r = rg * 8 + k;
+      const int r = rg * 2 + k / 4, col = cg * 4 + k % 4;
       if (r < nr && c0 + col < V) {
         float* o = out + (long)(t0 + r) * ldo + h * V + c0 + col;
         if (KIND == 0) {
@@ -351,8 +371,11 @@ TIS_EXPORT int tis_state_scan(int kind, const float* proj, long ldp, int q_off, 
   if (state_ld < tis_state_scan_floats(kind, H, D, V))
     return tis_fail("state_scan: a state line of %ld floats is too short for %ld", state_ld, tis_state_scan_floats(kind, H, D, V));
   int chunk = 16;
+  const int ns_built = (D + SC_R - 1) / SC_R <= 1 ? 1 : (D + SC_R - 1) / SC_R <= 2 ? 2 : (D + SC_R - 1) / SC_R <= 4 ? 4
+                       : (D + SC_R - 1) / SC_R <= 8 ? 8 : 16;
+  const size_t dp = (size_t)SC_R * ns_built;      // a token's row in LDS (see the kernel)
   auto bytes = [&](int c) {
-    return sizeof(float) * ((size_t)c * D * 2 + (kind == 0 ? (size_t)c * D : (size_t)c * 3) + (size_t)c * SC_VB +
+    return sizeof(float) * ((size_t)c * dp * 2 + (kind == 0 ? (size_t)c * dp : (size_t)c * 4) + (size_t)c * SC_VB +
                             (size_t)c * SC_R * (SC_VB + 1));
   };
   while (chunk > 1 && bytes(chunk) > SC_LDS_BYTES) chunk /= 2;
