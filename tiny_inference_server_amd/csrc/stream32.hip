@@ -29,7 +29,7 @@ __global__ __launch_bounds__(S32_THREADS) void embed_scale_kernel(const T* __res
 
 // r = alpha * x + sigmoid(gate + bias) * (s0 * y0 + s1 * y1);  out = r / sqrt(mean(r^2) + eps) * gain
 // y1 and gate may be null (one branch; no gate).
-template <typename T>
+template <typename T, int PER>      // PER: values a thread keeps in registers (width <= 256 * PER); 0: any width, through memory
 __global__ __launch_bounds__(S32_THREADS) void gated_postnorm_kernel(
     const float* __restrict__ x, const float* __restrict__ y0, long ld0, float s0, const float* __restrict__ y1, long ld1,
     float s1, const float* __restrict__ gate, long ldg, const float* __restrict__ bias, float alpha,
@@ -37,20 +37,45 @@ __global__ __launch_bounds__(S32_THREADS) void gated_postnorm_kernel(
   __shared__ float red[16];
   const long r = blockIdx.x;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+  float keep[PER > 0 ? PER : 1];
+  auto summed = [&](int c) {
     float y = s0 * y0[r * ld0 + c];
     if (y1) y += s1 * y1[r * ld1 + c];
     if (gate) y *= sigmoid_f(gate[r * ldg + c] + (bias ? bias[c] : 0.f));
-    const float v = alpha * x[r * D + c] + y;
-    out32[r * D + c] = v;
-    ss += v * v;
+    return alpha * x[r * D + c] + y;
+  };
+  if (PER > 0) {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int c = threadIdx.x + k * S32_THREADS;
+      keep[k] = c < D ? summed(c) : 0.f;
+      ss += keep[k] * keep[k];
+    }
+  } else {
+    for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+      const float v = summed(c);
+      out32[r * D + c] = v;
+      ss += v * v;
+    }
   }
-  ss = block_sum(ss, red);
+  ss = block_sum(ss, red);      // (the order of this sum depends on the width alone, whichever way the values are kept)
   const float inv = 1.f / sqrtf(ss / (float)D + eps);
-  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
-    const float v = out32[r * D + c] * inv * gain[c];
-    out32[r * D + c] = v;
-    if (outT) outT[r * D + c] = from_f<T>(v);
+  if (PER > 0) {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int c = threadIdx.x + k * S32_THREADS;
+      if (c < D) {
+        const float v = keep[k] * inv * gain[c];
+        out32[r * D + c] = v;
+        if (outT) outT[r * D + c] = from_f<T>(v);
+      }
+    }
+  } else {
+    for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+      const float v = out32[r * D + c] * inv * gain[c];
+      out32[r * D + c] = v;
+      if (outT) outT[r * D + c] = from_f<T>(v);
+    }
   }
 }
 
@@ -129,8 +154,16 @@ TIS_EXPORT int tis_gated_postnorm(int dtype, const float* x, const float* y0, lo
                                   float eps, float* out32, void* outT, int rows, int D, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || D < 1 || !x || !y0 || !gain || !out32) return tis_fail("gated_postnorm: bad arguments rows=%d width=%d", rows, D);
-  S32_DISPATCH((gated_postnorm_kernel<float><<<rows, S32_THREADS, 0, stream>>>(x, y0, ld0, s0, y1, ld1, s1, gate, ldg, bias, alpha, gain, eps, out32, (float*)outT, D)),
-               (gated_postnorm_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>(x, y0, ld0, s0, y1, ld1, s1, gate, ldg, bias, alpha, gain, eps, out32, (bf16*)outT, D)))
+#define S32_POSTNORM(T, PER)                                                                                           \
+  gated_postnorm_kernel<T, PER><<<rows, S32_THREADS, 0, stream>>>(x, y0, ld0, s0, y1, ld1, s1, gate, ldg, bias, alpha, gain, \
+                                                                  eps, out32, (T*)outT, D)
+#define S32_POSTNORM_BY_WIDTH(T)                         \
+  if (D <= 4 * S32_THREADS) { S32_POSTNORM(T, 4); }      \
+  else if (D <= 16 * S32_THREADS) { S32_POSTNORM(T, 16); } \
+  else { S32_POSTNORM(T, 0); }
+  S32_DISPATCH(S32_POSTNORM_BY_WIDTH(float), S32_POSTNORM_BY_WIDTH(bf16))
+#undef S32_POSTNORM_BY_WIDTH
+#undef S32_POSTNORM
   return tis_launch_status("gated_postnorm");
 }
 
