@@ -60,11 +60,14 @@ def _configs():
                         shared(with_mlp(gla(2, 12, 20, tau=5.0), 56), 0)], scale=3.5, alpha=2.2)
     # a window longer than any sequence of the tests, wide heads, a width that is no multiple of 8
     D = config(76, 150, [with_mlp(parallel(2, 2, 48, 80, 4096, 20, 2, 80, 36, base=1e6, scale=0.15), 120)], alpha=0.9)
-    return {"A": A, "B": B, "C": C, "D": D}
+    # heads as wide as a served model's (128 channels, values of 256 in the recurrences), keys and values of one size
+    e0 = with_mlp(parallel(4, 2, 128, 128, 100, 64, 2, 128, 256, base=5e5, scale=128 ** -0.5), 384)
+    E = config(256, 300, [e0, with_mlp(gla(2, 128, 256, tau=16.0), 320), shared(e0, 0)], scale=1.5, alpha=1.2)
+    return {"A": A, "B": B, "C": C, "D": D, "E": E}
 
 
 CONFIGS = _configs()
-RANK = {"A": 6, "B": 10, "C": 4, "D": 8}
+RANK = {"A": 6, "B": 10, "C": 4, "D": 8, "E": 16}
 
 
 def tensor_shapes(cfg, rank) -> Dict[str, tuple]:

@@ -211,6 +211,29 @@ def test_a_token_that_stands_out(name, distance, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_heads_of_served_sizes(dtype):
+    """Heads of 128 channels (the matrix-core attention kernels in bfloat16, eight state elements a thread in the
+    scans), prompts long enough for the scans to run in segments and for the window to pass, then decoded tokens;
+    alone and two requests together, the second cut into portions."""
+    cfg, w, w64 = model("E", seed=9)
+    reqs = {"a": H.random_ids(cfg["vocab"], 330, 1), "b": H.random_ids(cfg["vocab"], 215, 2)}
+    eng = engine_for(cfg, w, dtype)
+    got = FM.run_trace(eng, H.tail_decode_trace(reqs, tail=12))
+    worst = FM.worst_error("E", cfg, w64, reqs, got)
+    assert worst[0] <= TOL[dtype], worst
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": reqs["a"][:300], "want": list(range(0, 300, 7))},
+                                     {"id": "b", "tokens": reqs["b"][:3], "want": [0, 1, 2]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": reqs["a"][300:301], "want": [0]},
+                                     {"id": "b", "tokens": reqs["b"][3:200], "want": list(range(0, 197, 5))}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": reqs["a"][301:], "want": list(range(29))},
+                                     {"id": "b", "tokens": reqs["b"][200:], "want": list(range(15))}], "end": ["a", "b"]}]
+    got = FM.run_trace(eng, steps)
+    worst = FM.worst_error("E", cfg, w64, reqs, got)
+    assert worst[0] <= TOL[dtype], worst
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_through_captured_steps(dtype):
     """Three requests decode 150 tokens together, past every window and over many page borders; steps of single tokens
     are replayed from captured graphs, and every replay is checked."""
