@@ -63,11 +63,15 @@ def _configs():
     # heads as wide as a served model's (128 channels, values of 256 in the recurrences), keys and values of one size
     e0 = with_mlp(parallel(4, 2, 128, 128, 100, 64, 2, 128, 256, base=5e5, scale=128 ** -0.5), 384)
     E = config(256, 300, [e0, with_mlp(gla(2, 128, 256, tau=16.0), 320), shared(e0, 0)], scale=1.5, alpha=1.2)
-    return {"A": A, "B": B, "C": C, "D": D, "E": E}
+    # keys and values of one size that no matrix-core kernel takes (24 channels), no rotation and no rotary base
+    f0 = with_mlp(parallel(3, 3, 24, 24, 13, 0, 2, 10, 12, scale=0.3), 40)
+    del f0["mixer"]["left"]["rot"]["base"]
+    F = config(48, 77, [with_mlp(gla(2, 16, 8, tau=2.0), 64), f0], scale=1.0, alpha=1.4)
+    return {"A": A, "B": B, "C": C, "D": D, "E": E, "F": F}
 
 
 CONFIGS = _configs()
-RANK = {"A": 6, "B": 10, "C": 4, "D": 8, "E": 16}
+RANK = {"A": 6, "B": 10, "C": 4, "D": 8, "E": 16, "F": 3}
 
 
 def tensor_shapes(cfg, rank) -> Dict[str, tuple]:

@@ -55,8 +55,8 @@ def windowed_attention(h, w, pre, p, eps):
     q = rms_norm(q, eps, w[pre + "q.norm"])
     k = rms_norm(k, eps, w[pre + "k.norm"])
     pos = torch.arange(T)
-    q = rotate_pairs(q, pos, p["rot"]["dims"], p["rot"]["base"])
-    k = rotate_pairs(k, pos, p["rot"]["dims"], p["rot"]["base"])
+    q = rotate_pairs(q, pos, p["rot"]["dims"], p["rot"].get("base"))
+    k = rotate_pairs(k, pos, p["rot"]["dims"], p["rot"].get("base"))
     v = rms_norm(v, eps)
     size = p["mask"]["size"]
     out = torch.zeros(T, H, V, dtype=F64)

@@ -135,7 +135,7 @@ def test_attention_with_keys_and_values_of_different_sizes(dtype, Hq, G, kd, vd,
 @pytest.mark.parametrize("segment", [64, 8, 5])
 @pytest.mark.parametrize("kind,Hh,D,V", [("decay", 3, 20, 24), ("gated_max", 2, 24, 40), ("decay", 1, 130, 17),
                                          ("gated_max", 5, 7, 16), ("gated_max", 1, 256, 70), ("gated_max", 2, 64, 130),
-                                         ("decay", 2, 128, 64)])
+                                         ("decay", 2, 128, 64), ("gated_max", 2, 128, 128), ("decay", 1, 96, 192)])
 def test_state_scan_against_the_token_by_token_rule(kind, Hh, D, V, segment):
     """Portions of three requests in one call, then their next portions and single tokens in further calls, on state
     lines that start from what an earlier owner left: every result and the final state against plain torch. With

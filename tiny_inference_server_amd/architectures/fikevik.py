@@ -41,7 +41,7 @@ def _gla(cfg, m, pre):
 def _left(cfg, m, pre):
     params = {"width": cfg.width, "n_heads": m["heads"], "n_kv_heads": m["kv_heads"], "key_dim": m["dim"],
               "value_dim": m["vdim"], "window": m["mask"]["size"], "rot_dims": m["rot"]["dims"],
-              "rot_base": m["rot"]["base"], "scale": m["scale"], "eps": cfg.norm_eps}
+              "rot_base": m["rot"].get("base", 1.0), "scale": m["scale"], "eps": cfg.norm_eps}
     names = {k: pre + k for k in ("q", "k", "v", "o", "temp")}
     names.update(q_norm=pre + "q.norm", k_norm=pre + "k.norm")
     return PartSpec("mixer", "windowed_qknorm_attention", params, names)

@@ -64,7 +64,8 @@ def _check_layer(i, entry, n_layers):
         _number(left, "scale", lw, float)
         _number(left.get("mask"), "size", lw + ".mask", int, 1)
         dims = _number(left.get("rot"), "dims", lw + ".rot", int, 0)
-        _number(left.get("rot"), "base", lw + ".rot", float)
+        if dims:
+            _need(_number(left.get("rot"), "base", lw + ".rot", float) > 0, f"{lw}.rot.base must be positive")
         _need(dims % 2 == 0 and dims <= left["dim"], f"{lw}.rot.dims {dims}: an even number, at most dim {left['dim']}")
         _check_recurrent(right, where + ".mixer.right")
         _number(right, "gate_cap", where + ".mixer.right", float)

@@ -49,20 +49,25 @@ struct SegArgs {
   float* aux;
 };
 
-template <int KIND, int NS, bool SEG>
+// VB value channels a workgroup, R = 256 / VB threads a column. A request's state line keeps n and m once per 16 value
+// channels, so the walk in order runs with VB = 16; segments keep n and m once per head and may take 64 channels a
+// workgroup, which loads a head's q, k and decays a quarter as often.
+template <int KIND, int NS, bool SEG, int VB>
 __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
     const float* __restrict__ proj, long ldp, int q_off, int k_off, int v_off, float q_scale,
     const float* __restrict__ decay, long ldd, int i_off, int f_off, const float* __restrict__ bias_i,
     const float* __restrict__ bias_f, float cap, float* __restrict__ state, long state_ld,
     const int* __restrict__ cu_rows, const int* __restrict__ seq_slots, float* __restrict__ out, long ldo, int H, int D,
     int V, int n_vb, int chunk, SegArgs sg) {
+  static_assert(SEG || VB == SC_VB, "a state line keeps n and m per 16 value channels");
+  constexpr int R = SC_THREADS / VB;
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int DP = SC_R * NS;                      // a token's row in LDS: the head's channels, then zeros
+  constexpr int DP = R * NS;                         // a token's row in LDS: the head's channels, then zeros
   float* sq = lds;                                   // [chunk][DP]
   float* sk = sq + chunk * DP;                       // [chunk][DP]
   float* sa = sk + chunk * DP;                       // kind 0: [chunk][DP] decays; kind 1: [chunk][4] gates i, f and m
   float* sv = sa + (KIND == 0 ? chunk * DP : chunk * 4);  // [chunk][VB]
-  float* part = sv + chunk * SC_VB;                  // [chunk][R][VB + 1]
+  float* part = sv + chunk * VB;                     // [chunk][R][VB + 1]
 
   const int seq = SEG ? blockIdx.x / sg.segments : blockIdx.x, h = blockIdx.y, vb = blockIdx.z, t = threadIdx.x;
   int r0 = cu_rows[seq], r1 = cu_rows[seq + 1];
@@ -75,8 +80,8 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
   float* S = st + (long)h * (SEG ? (long)D * V + D + 2 : (long)D * V);
   // kind 1: n [D], then m; once per block of value channels in a request's state line, once per head in a segment's
   float* nm = SEG ? S + (long)D * V : st + (long)H * D * V + ((long)h * n_vb + vb) * (D + 1);
-  const int j = t % SC_VB, s = t / SC_VB;
-  const int col = vb * SC_VB + j;
+  const int j = t % VB, s = t / VB;
+  const int col = vb * VB + j;
   const bool col_ok = col < V;
 
   float Sreg[NS], nreg[NS], creg[NS];
@@ -101,9 +106,9 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
       sk[idx] = in ? row[k_off + h * D + i] : 0.f;
       if (KIND == 0) sa[idx] = in ? decay[(long)(c0 + c) * ldd + h * D + i] : 0.f;
     }
-    for (int idx = t; idx < nc * SC_VB; idx += SC_THREADS) {
-      const int c = idx / SC_VB, jj = idx - c * SC_VB;
-      sv[idx] = (vb * SC_VB + jj < V) ? proj[(long)(c0 + c) * ldp + v_off + h * V + vb * SC_VB + jj] : 0.f;
+    for (int idx = t; idx < nc * VB; idx += SC_THREADS) {
+      const int c = idx / VB, jj = idx - c * VB;
+      sv[idx] = (vb * VB + jj < V) ? proj[(long)(c0 + c) * ldp + v_off + h * V + vb * VB + jj] : 0.f;
     }
     if (KIND == 1 && t < nc) {
       const float* row = proj + (long)(c0 + t) * ldp;
@@ -122,64 +127,63 @@ __global__ __launch_bounds__(SC_THREADS) void state_scan_kernel(
         m = m_new;
         fsum += gf;
       }
-      const float vj = sv[c * SC_VB + j];
+      const float vj = sv[c * VB + j];
       float acc = 0.f, nq = 0.f;
-      float kk[NS], qq[NS], aa[NS];
       const int at = c * DP + s * NS;
-      if (NS % 4 == 0) {
-#pragma unroll
-        for (int e = 0; e < NS; e += 4) {
-          *reinterpret_cast<float4*>(kk + e) = *reinterpret_cast<const float4*>(sk + at + e);
-          *reinterpret_cast<float4*>(qq + e) = *reinterpret_cast<const float4*>(sq + at + e);
-          if (KIND == 0) *reinterpret_cast<float4*>(aa + e) = *reinterpret_cast<const float4*>(sa + at + e);
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < NS; ++e) {
-          kk[e] = sk[at + e];
-          qq[e] = sq[at + e];
-          if (KIND == 0) aa[e] = sa[at + e];
-        }
-      }
       // (channels beyond the head's are zeros in k and q: their state stays zero and adds nothing)
+      constexpr int STEP = NS % 4 == 0 ? 4 : 1;      // a thread reads its channels in 16-byte pieces where they allow
 #pragma unroll
-      for (int e = 0; e < NS; ++e) {
-        if (KIND == 0) {
-          Sreg[e] = aa[e] * Sreg[e] + kk[e] * vj;
-          if (SEG) creg[e] *= aa[e];
+      for (int e0 = 0; e0 < NS; e0 += STEP) {
+        float kk[STEP], qq[STEP], aa[STEP];
+        if (STEP == 4) {
+          *reinterpret_cast<float4*>(kk) = *reinterpret_cast<const float4*>(sk + at + e0);
+          *reinterpret_cast<float4*>(qq) = *reinterpret_cast<const float4*>(sq + at + e0);
+          if (KIND == 0) *reinterpret_cast<float4*>(aa) = *reinterpret_cast<const float4*>(sa + at + e0);
         } else {
-          Sreg[e] = keep * Sreg[e] + take * (kk[e] * vj);
-          nreg[e] = keep * nreg[e] + take * kk[e];
-          nq += nreg[e] * qq[e];
+          kk[0] = sk[at + e0];
+          qq[0] = sq[at + e0];
+          if (KIND == 0) aa[0] = sa[at + e0];
         }
-        acc += Sreg[e] * qq[e];
+#pragma unroll
+        for (int u = 0; u < STEP; ++u) {
+          const int e = e0 + u;
+          if (KIND == 0) {
+            Sreg[e] = aa[u] * Sreg[e] + kk[u] * vj;
+            if (SEG) creg[e] *= aa[u];
+          } else {
+            Sreg[e] = keep * Sreg[e] + take * (kk[u] * vj);
+            nreg[e] = keep * nreg[e] + take * kk[u];
+            nq += nreg[e] * qq[u];
+          }
+          acc += Sreg[e] * qq[u];
+        }
       }
       if (KIND == 0 && SEG && vb == 0 && j == 0) {
 #pragma unroll
         for (int e = 0; e < NS; ++e)
           if (s * NS + e < D) sg.cum[(long)(c0 + c) * H * D + h * D + s * NS + e] = creg[e];
       }
-      part[(c * SC_R + s) * (SC_VB + 1) + j] = acc;
+      part[(c * R + s) * (VB + 1) + j] = acc;
       if (KIND == 1) {
-        if (j == 0) part[(c * SC_R + s) * (SC_VB + 1) + SC_VB] = nq;
+        if (j == 0) part[(c * R + s) * (VB + 1) + VB] = nq;
         if (t == 0) sa[c * 4 + 2] = m;
         if (SEG && t == 0 && vb == 0) sg.aux[((long)(c0 + c) * H + h) * 3 + 1] = fsum;
       }
     }
     __syncthreads();
-    for (int idx = t; idx < nc * SC_VB; idx += SC_THREADS) {
-      const int c = idx / SC_VB, jj = idx - c * SC_VB;
+    for (int idx = t; idx < nc * VB; idx += SC_THREADS) {
+      const int c = idx / VB, jj = idx - c * VB;
       float o = 0.f, nq = 0.f;
-      for (int ss = 0; ss < SC_R; ++ss) {
-        o += part[(c * SC_R + ss) * (SC_VB + 1) + jj];
-        if (KIND == 1) nq += part[(c * SC_R + ss) * (SC_VB + 1) + SC_VB];
+      for (int ss = 0; ss < R; ++ss) {
+        o += part[(c * R + ss) * (VB + 1) + jj];
+        if (KIND == 1) nq += part[(c * R + ss) * (VB + 1) + VB];
       }
       if (KIND == 1 && !SEG) o /= fmaxf(fabsf(nq), expf(-sa[c * 4 + 2])) + 1e-6f;
       if (KIND == 1 && SEG && vb == 0 && jj == 0) {
         sg.aux[((long)(c0 + c) * H + h) * 3] = sa[c * 4 + 2];
         sg.aux[((long)(c0 + c) * H + h) * 3 + 2] = nq;
       }
-      if (vb * SC_VB + jj < V) out[(long)(c0 + c) * ldo + h * V + vb * SC_VB + jj] = o;
+      if (vb * VB + jj < V) out[(long)(c0 + c) * ldo + h * V + vb * VB + jj] = o;
     }
   }
 #pragma unroll
@@ -305,25 +309,37 @@ __global__ __launch_bounds__(SC_THREADS) void segment_outputs_kernel(const float
   }
 }
 
+static constexpr int SC_WIDE_VB = 64;      // value channels of a workgroup that walks a segment, where the sizes allow
+
 template <int KIND>
-static int launch_scan(int ns, dim3 grid, size_t lds, hipStream_t stream, const float* proj, long ldp, int q_off, int k_off,
+static int launch_scan(bool wide, int ns, dim3 grid, size_t lds, hipStream_t stream, const float* proj, long ldp, int q_off, int k_off,
                        int v_off, float q_scale, const float* decay, long ldd, int i_off, int f_off, const float* bias_i,
                        const float* bias_f, float cap, float* state, long state_ld, const int* cu_rows,
                        const int* seq_slots, float* out, long ldo, int H, int D, int V, int n_vb, int chunk, SegArgs sg) {
 #define SC_LAUNCH(NS)                                                                                                   \
   if (sg.segments)                                                                                                      \
-    state_scan_kernel<KIND, NS, true><<<grid, SC_THREADS, lds, stream>>>(                                               \
+    state_scan_kernel<KIND, NS, true, SC_VB><<<grid, SC_THREADS, lds, stream>>>(                                        \
         proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off, bias_i, bias_f, cap, state, state_ld,        \
         cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);                                                        \
   else                                                                                                                  \
-    state_scan_kernel<KIND, NS, false><<<grid, SC_THREADS, lds, stream>>>(                                              \
+    state_scan_kernel<KIND, NS, false, SC_VB><<<grid, SC_THREADS, lds, stream>>>(                                       \
         proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off, bias_i, bias_f, cap, state, state_ld,        \
         cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg)
+#define SC_LAUNCH_WIDE(NS)                                                                                              \
+  state_scan_kernel<KIND, NS, true, SC_WIDE_VB><<<grid, SC_THREADS, lds, stream>>>(                                     \
+      proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off, bias_i, bias_f, cap, state, state_ld, cu_rows, \
+      seq_slots, out, ldo, H, D, V, n_vb, chunk, sg)
+  if (wide) {
+    if (ns <= 8) { SC_LAUNCH_WIDE(8); }
+    else if (ns <= 16) { SC_LAUNCH_WIDE(16); }
+    else { SC_LAUNCH_WIDE(32); }
+  } else
   if (ns <= 1) { SC_LAUNCH(1); }
   else if (ns <= 2) { SC_LAUNCH(2); }
   else if (ns <= 4) { SC_LAUNCH(4); }
   else if (ns <= 8) { SC_LAUNCH(8); }
   else { SC_LAUNCH(16); }
+#undef SC_LAUNCH_WIDE
 #undef SC_LAUNCH
   if (tis_launch_status("state_scan")) return -1;
   if (!sg.segments) return 0;
@@ -370,13 +386,17 @@ TIS_EXPORT int tis_state_scan(int kind, const float* proj, long ldp, int q_off, 
   if (n_vb > 65535) return tis_fail("state_scan: %d value channels exceed the grid", V);
   if (state_ld < tis_state_scan_floats(kind, H, D, V))
     return tis_fail("state_scan: a state line of %ld floats is too short for %ld", state_ld, tis_state_scan_floats(kind, H, D, V));
+  // segments of heads with up to 128 key channels and whole blocks of 64 value channels: 64 channels a workgroup
+  const bool wide = segments > 0 && V % SC_WIDE_VB == 0 && D <= 32 * (SC_THREADS / SC_WIDE_VB);
+  const int vb_cols = wide ? SC_WIDE_VB : SC_VB, col_threads = SC_THREADS / vb_cols;
   int chunk = 16;
-  const int ns_built = (D + SC_R - 1) / SC_R <= 1 ? 1 : (D + SC_R - 1) / SC_R <= 2 ? 2 : (D + SC_R - 1) / SC_R <= 4 ? 4
+  const int ns_need = (D + col_threads - 1) / col_threads;
+  const int ns_built = wide ? (ns_need <= 8 ? 8 : ns_need <= 16 ? 16 : 32) : (D + SC_R - 1) / SC_R <= 1 ? 1 : (D + SC_R - 1) / SC_R <= 2 ? 2 : (D + SC_R - 1) / SC_R <= 4 ? 4
                        : (D + SC_R - 1) / SC_R <= 8 ? 8 : 16;
-  const size_t dp = (size_t)SC_R * ns_built;      // a token's row in LDS (see the kernel)
+  const size_t dp = (size_t)col_threads * ns_built;      // a token's row in LDS (see the kernel)
   auto bytes = [&](int c) {
-    return sizeof(float) * ((size_t)c * dp * 2 + (kind == 0 ? (size_t)c * dp : (size_t)c * 4) + (size_t)c * SC_VB +
-                            (size_t)c * SC_R * (SC_VB + 1));
+    return sizeof(float) * ((size_t)c * dp * 2 + (kind == 0 ? (size_t)c * dp : (size_t)c * 4) + (size_t)c * vb_cols +
+                            (size_t)c * col_threads * (vb_cols + 1));
   };
   while (chunk > 1 && bytes(chunk) > SC_LDS_BYTES) chunk /= 2;
   if (bytes(chunk) > SC_LDS_BYTES) return tis_fail("state_scan: %d key channels do not fit the chunk buffers", D);
@@ -393,11 +413,11 @@ TIS_EXPORT int tis_state_scan(int kind, const float* proj, long ldp, int q_off, 
     if (sizeof(float) * ((size_t)D * SG_COLS + (size_t)SG_ROWS * (D + 1) + SG_ROWS) > 64 * 1024)
       return tis_fail("state_scan: %d key channels do not fit the segment kernels (see tis_state_scan_segmentable)", D);
   }
-  dim3 grid(segments > 0 ? n_seqs * segments : n_seqs, H, n_vb);
-  const int ns = (D + SC_R - 1) / SC_R;
+  dim3 grid(segments > 0 ? n_seqs * segments : n_seqs, H, (V + vb_cols - 1) / vb_cols);
+  const int ns = ns_need;
   if (kind == 0)
-    return launch_scan<0>(ns, grid, bytes(chunk), stream, proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off,
+    return launch_scan<0>(wide, ns, grid, bytes(chunk), stream, proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off,
                           bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);
-  return launch_scan<1>(ns, grid, bytes(chunk), stream, proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off,
+  return launch_scan<1>(wide, ns, grid, bytes(chunk), stream, proj, ldp, q_off, k_off, v_off, q_scale, decay, ldd, i_off, f_off,
                         bias_i, bias_f, cap, state, state_ld, cu_rows, seq_slots, out, ldo, H, D, V, n_vb, chunk, sg);
 }
