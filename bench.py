@@ -294,11 +294,11 @@ def fikevik_config(width, heads, kv_heads, ff, layers, vocab, window=1024):
     from tiny_inference_server_amd.config import config_from_dict
     par = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
            "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "mask": {"size": window},
-                              "rot": {"dims": 64, "base": 500000.0}, "scale": 128 ** -0.5},
-                     "right": {"heads": heads // 2, "dim": 128, "vdim": 256, "gate_cap": 15.0},
+                              "rot": {"dims": 64, "base": 1000000.0}, "scale": 128 ** -0.5},
+                     "right": {"heads": heads // 2, "dim": 128, "vdim": 256, "gate_cap": 12.0},
                      "left_scale": 1.0, "right_scale": 1.0}}
     gla = {"type": "gla", "mlp": {"kind": "dense", "ff": ff},
-           "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "tau": 16.0, "rank": 16}}
+           "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "tau": 8.0, "rank": 32}}
     return config_from_dict({"architecture": "Fikevik", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
                              "norm": {"eps": 1e-5}, "postln_alpha": 1.0,
                              "layers": [par if i % 2 == 0 else gla for i in range(layers)]})

@@ -61,8 +61,8 @@ def _configs():
     # a window longer than any sequence of the tests, wide heads, a width that is no multiple of 8
     D = config(76, 150, [with_mlp(parallel(2, 2, 48, 80, 4096, 20, 2, 80, 36, base=1e6, scale=0.15), 120)], alpha=0.9)
     # heads as wide as a served model's (128 channels, values of 256 in the recurrences), keys and values of one size
-    e0 = with_mlp(parallel(4, 2, 128, 128, 100, 64, 2, 128, 256, base=5e5, scale=128 ** -0.5), 384)
-    E = config(256, 300, [e0, with_mlp(gla(2, 128, 256, tau=16.0), 320), shared(e0, 0)], scale=1.5, alpha=1.2)
+    e0 = with_mlp(parallel(4, 2, 128, 128, 100, 64, 2, 128, 256, base=2e5, scale=128 ** -0.5), 448)
+    E = config(320, 300, [e0, with_mlp(gla(2, 128, 256, tau=12.0), 352), shared(e0, 0)], scale=1.5, alpha=1.2)
     # keys and values of one size that no matrix-core kernel takes (24 channels), no rotation and no rotary base
     f0 = with_mlp(parallel(3, 3, 24, 24, 13, 0, 2, 10, 12, scale=0.3), 40)
     del f0["mixer"]["left"]["rot"]["base"]

@@ -234,6 +234,24 @@ def test_heads_of_served_sizes(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_step_that_repeats_is_replayed(dtype):
+    """Prompts of one length, one after the other: from its third occurrence the step (attention over the pages, the
+    scans in segments with their workspace, the state slot of whoever was there before) is replayed from a captured
+    graph; every run is checked, with other work between the replays."""
+    cfg, w, w64 = model("E", seed=9)
+    eng = engine_for(cfg, w, dtype, max_requests=2)
+    other = H.random_ids(cfg["vocab"], 40, 77)
+    for k in range(6):
+        ids = H.random_ids(cfg["vocab"], 200, 30 + k)
+        got = FM.run_trace(eng, [{"step": 0, "entries": [{"id": "p", "tokens": ids, "want": [0, 64, 127, 128, 199]}],
+                                  "end": ["p"]}])
+        assert FM.worst_error(("E", k), cfg, w64, {"p": ids}, got)[0] <= TOL[dtype]
+        got = FM.run_trace(eng, H.portions_trace({"o": other}, sizes=(7, 1, 12)))
+        assert FM.worst_error("Eo", cfg, w64, {"o": other}, got)[0] <= TOL[dtype]
+    assert eng.graph_replays >= 3
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_through_captured_steps(dtype):
     """Three requests decode 150 tokens together, past every window and over many page borders; steps of single tokens
     are replayed from captured graphs, and every replay is checked."""
