@@ -175,12 +175,14 @@ class TorchOps:
         return torch.exp(torch.nn.functional.logsigmoid(z) / tau)
 
     def attention_prepare(self, proj, q_off, k_off, v_off, positions, write_slots, plane, n_heads, n_kv_heads, key_dim,
-                          value_dim, page_size, q_gain, k_gain, q_factor, freqs, rot_dims, eps, write_cache=True):
+                          value_dim, page_size, q_gain=None, k_gain=None, q_factor=None, freqs=None, rot_dims=0, eps=0.0,
+                          write_cache=True, value_norm=True, q_bias=None, k_bias=None, v_bias=None, temp_coef=0.0,
+                          temp_every=1):
         n = proj.shape[0]
         H, G, kd, vd = n_heads, n_kv_heads, key_dim, value_dim
 
         def normed(x, gain):
-            return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain
+            return x if gain is None else x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * gain
 
         def turned(x):
             if not rot_dims:
@@ -193,10 +195,19 @@ class TorchOps:
             y[..., 1:rot_dims:2] = b * c + a * s
             return y
 
-        q = turned(normed(proj[:, q_off:q_off + H * kd].float().reshape(n, H, kd), q_gain)) * q_factor[None, :, None]
+        def part(off, heads, dim, bias):
+            x = proj[:, off:off + heads * dim].float()
+            return (x + bias if bias is not None else x).reshape(n, heads, dim)
+
+        q = turned(normed(part(q_off, H, kd, q_bias), q_gain))
+        if q_factor is not None:
+            q = q * q_factor[None, :, None]
+        if temp_coef:
+            p1 = torch.div(positions.long() + 1, temp_every, rounding_mode="floor").float()
+            q = q * (1.0 + temp_coef * torch.log(p1 + 1.0))[:, None, None]
         if write_cache:
-            k = turned(normed(proj[:, k_off:k_off + G * kd].float().reshape(n, G, kd), k_gain)).to(plane.dtype)
-            v = normed(proj[:, v_off:v_off + G * vd].float().reshape(n, G, vd), 1.0).to(plane.dtype)
+            k = turned(normed(part(k_off, G, kd, k_bias), k_gain)).to(plane.dtype)
+            v = normed(part(v_off, G, vd, v_bias), 1.0 if value_norm else None).to(plane.dtype)
             pages = plane.view(plane.shape[0], -1)
             page, off = write_slots.long() // page_size, write_slots.long() % page_size
             keys = pages[:, :G * page_size * kd].view(-1, G, page_size, kd)
@@ -205,15 +216,48 @@ class TorchOps:
             vals[page, :, :, off] = v
         return q.reshape(n, H * kd).to(self.dtype)
 
+    def latent_prepare(self, proj, q_off, c_off, positions, write_slots, plane, n_heads, dim, rot_dim, rank, page_size,
+                       gain, freqs, rot_dims, eps, write_cache=True):
+        n, H, D, R, C = proj.shape[0], n_heads, dim, rot_dim, rank
+
+        def turned(x):                    # [n, ..., R]
+            if not rot_dims:
+                return x
+            ang = positions.float()[:, None] * freqs[None, :]
+            shape = (n,) + (1,) * (x.dim() - 2) + (rot_dims // 2,)
+            c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+            a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+            y = x.clone()
+            y[..., 0:rot_dims:2] = a * c - b * s
+            y[..., 1:rot_dims:2] = b * c + a * s
+            return y
+
+        qh = proj[:, q_off:q_off + H * (D + R)].float().view(n, H, D + R)
+        q = torch.zeros(n, H, C + R, dtype=self.dtype, device=proj.device)
+        q[..., C:] = turned(qh[..., D:]).to(self.dtype)
+        q_plain = qh[..., :D].reshape(n, H * D).to(self.dtype)
+        if D == 0:
+            q_plain = torch.zeros(n, H, dtype=self.dtype, device=proj.device)
+        if write_cache:
+            c = proj[:, c_off:c_off + C].float()
+            c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * gain
+            key = torch.cat((c, turned(proj[:, c_off + C:c_off + C + R].float())), dim=-1).to(plane.dtype)
+            pages = plane.view(plane.shape[0], page_size, C + R)
+            pages[write_slots.long() // page_size, write_slots.long() % page_size] = key
+        return q.view(n, H * (C + R)), q_plain
+
     def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
-                           scale=None):
+                           scale=None, sink=False, gate=None, latent=False):
         n = q.shape[0]
         H, G, kd, vd = n_heads, n_kv_heads, key_dim, value_dim
         scale = scale if scale is not None else kd ** -0.5
         tables = batch.block_tables[group]
         pages = plane.view(plane.shape[0], -1)
-        keys = pages[:, :G * page_size * kd].view(-1, G, page_size, kd)
-        vals = pages[:, G * page_size * kd:].view(-1, G, vd, page_size)
+        if latent:
+            keys = pages.view(-1, 1, page_size, kd)
+        else:
+            keys = pages[:, :G * page_size * kd].view(-1, G, page_size, kd)
+            vals = pages[:, G * page_size * kd:].view(-1, G, vd, page_size)
         out = torch.zeros(n, H * vd, dtype=torch.float32, device=q.device)
         pos, seq = batch.positions.tolist(), batch.row_seq.tolist()
         for r in range(n):
@@ -221,12 +265,81 @@ class TorchOps:
             js = torch.arange(max(0, p - window + 1) if window > 0 else 0, p + 1)
             pg = tables[seq[r]].long()[js // page_size]
             k = keys[pg, :, js % page_size].float()          # [keys, G, kd]
-            v = vals[pg, :, :, js % page_size].float()       # [keys, G, vd]
+            v = k[..., :vd] if latent else vals[pg, :, :, js % page_size].float()       # [keys, G, vd]
             qr = q[r].float().view(H, kd)
             for h in range(H):
-                w = torch.softmax((k[:, h // (H // G)] @ qr[h]) * scale, dim=0)
-                out[r, h * vd:(h + 1) * vd] = w @ v[:, h // (H // G)]
+                sc = (k[:, h // (H // G)] @ qr[h]) * scale
+                if sink:
+                    w = torch.softmax(torch.cat((sc, sc.new_zeros(1))), dim=0)[:-1]
+                else:
+                    w = torch.softmax(sc, dim=0)
+                o = w @ v[:, h // (H // G)]
+                if gate is not None:
+                    o = o * torch.sigmoid(gate[r, h].float())
+                out[r, h * vd:(h + 1) * vd] = o
         return out.to(q.dtype)
+
+    # ---- a residual stream in 32-bit, norm before the sublayer ------------------------------------------------
+    def layernorm32(self, x32, gain, bias, eps):
+        mu = x32.mean(-1, keepdim=True)
+        var = ((x32 - mu) ** 2).mean(-1, keepdim=True)
+        y = (x32 - mu) / torch.sqrt(var + eps) * gain
+        return (y + bias if bias is not None else y).to(self.dtype)
+
+    def residual_norm(self, x32, y=None, y_rms=None, copy=False, norm=None):
+        if y is not None:
+            y = y.float()[:, :x32.shape[1]]
+            if y_rms is not None:
+                y = y / torch.sqrt((y * y).mean(-1, keepdim=True) + y_rms[1]) * y_rms[0]
+            x32 += y
+        normed = None
+        if norm is not None:
+            kind, gain, bias, eps = norm
+            normed = self.layernorm32(x32, gain, bias, eps) if kind == "layer" else self.rmsnorm32(x32, gain, eps)
+        cp = (x32 if self.dtype == torch.float32 else x32.to(self.dtype)) if copy else None
+        return x32, cp, normed
+
+    @staticmethod
+    def _act(z, act):
+        if act == "gelu_tanh":
+            return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+        return z * torch.sigmoid(z) if act == "silu" else torch.sigmoid(z)
+
+    def gate_table(self, z, table, tokens, act):
+        return (self._act(z.float(), act) * table[tokens.long()].float()).to(self.dtype)
+
+    def activate32(self, z, act):
+        z.copy_(self._act(z, act))
+        return z
+
+    # ---- products in groups ----------------------------------------------------------------------------------
+    def heads_linear(self, x, w, out, out_group, out_offset=0):
+        H, N, K = w.shape
+        y = torch.einsum("rhk,hnk->rhn", x.float().view(x.shape[0], H, K), w.float())
+        for h in range(H):
+            out[:, out_offset + h * out_group:out_offset + h * out_group + N] = y[:, h].to(out.dtype)
+        return out
+
+    def route_topk(self, z, correction, scale, top):
+        s = torch.softmax(z.float(), dim=-1)
+        choice = s + correction if correction is not None else s
+        ids = torch.topk(choice, top, dim=-1).indices
+        return ids.to(torch.int32), torch.gather(s, 1, ids) * scale
+
+    def routed_experts(self, x, ids, weights, w_up, w_down, act="gelu_erf"):
+        E = w_up.shape[0] if w_up is not None else 0
+        xf = x.float()
+        out = torch.zeros_like(xf)
+        for r in range(x.shape[0]):
+            for k in range(ids.shape[1]):
+                e = int(ids[r, k])
+                if e >= E:
+                    y = xf[r]
+                else:
+                    hid = torch.nn.functional.gelu(w_up[e].float() @ xf[r]).to(self.dtype).float()
+                    y = w_down[e].float() @ hid
+                out[r] += weights[r, k] * y
+        return out
 
     @staticmethod
     def state_scan_floats(kind, n_heads, dim, vdim):

@@ -2,3 +2,4 @@ from .model_config import (ARCHITECTURES, Architecture, ConfigError, GqaMtpConfi
                            save_config)
 from .registry import Registry
 from .fikevik_config import FikevikConfig
+from .fipuzen_config import FipuzenConfig

@@ -1,11 +1,14 @@
 // Softmax attention whose keys and values differ in size, over a paged cache, with a sliding window: the step before
-// it (per-head RMS norm of queries and keys, rotation of the first channels in interleaved pairs, a factor per query
-// head, unit-RMS values, the write into the pages) and the attention itself.
+// it (biases, per-head RMS norm of queries and keys, rotation of the first channels in interleaved pairs, a factor per
+// query head and one that grows with the position, unit-RMS values, the write into the pages: each optional), the same
+// step for keys and values that are one shared latent, and the attention itself, with an optional sink in the softmax
+// and an optional gate per head on the result.
 //
 // A page of `page_size` slots holds, for each key/value head, the keys as [slot][key size] and then, after the keys
 // of all heads, the values transposed as [value size][slot]. With equal sizes that is the layout the other attention
-// kernels read. The row at position p sees the keys at [max(0, p - window + 1), p] (window 0: all), found through the
-// request's block table; keys outside are never read, so what a reused page holds cannot reach a result.
+// kernels read. Pages of a latent hold keys only; the values are the keys' first channels. The row at position p sees
+// the keys at [max(0, p - window + 1), p] (window 0: all), found through the request's block table; keys outside are
+// never read, so what a reused page holds cannot reach a result.
 // Norms, angles, scores, the softmax and the weighted sum are 32-bit; `T` is the type of queries and pages.
 #include "common.h"
 
@@ -13,16 +16,32 @@ TIS_DEFINE_LAST_ERROR(tis_attention_window)
 
 static constexpr int AW_THREADS = 256;
 static constexpr int AW_CHUNK = 1024;
-static constexpr int AW_MAX_DIM = 256;
+static constexpr int AW_MAX_DIM = 1024;
+static constexpr int AW_PER = AW_MAX_DIM / AW_THREADS;   // value channels a thread may own
+
+// What the step before attention may do beyond copying: every pointer may be null and every count zero.
+struct PrepareArgs {
+  const float* q_bias;     // [H * KD], added to the projections
+  const float* k_bias;     // [G * KD]
+  const float* v_bias;     // [G * VD]
+  const float* q_gain;     // [KD]: RMS norm of every query head with this gain (null: no norm)
+  const float* k_gain;     // [KD]
+  const float* q_factor;   // [H]: a factor per query head
+  const float* freqs;      // [rot_dims / 2]: angle = position * freqs[pair], pairs (2i, 2i+1) of the first rot_dims channels
+  int rot_dims;
+  float eps;
+  int value_norm;          // values are divided by their root mean square
+  float temp_coef;         // queries times 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1); 0: none
+  int temp_every;
+};
 
 // grid (rows, H + 2 G), one wave each: unit u < H is a query head, u < H + G a key head, else a value head.
 // proj holds the projections of a row in 32-bit: queries at q_off, keys at k_off, values at v_off.
 template <typename T>
 __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
     const float* __restrict__ proj, long ldp, int q_off, int k_off, int v_off, const int* __restrict__ positions,
-    const int* __restrict__ write_slots, T* __restrict__ plane, T* __restrict__ q_out, long ldq,
-    const float* __restrict__ q_gain, const float* __restrict__ k_gain, const float* __restrict__ q_factor,
-    const float* __restrict__ freqs, int rot_dims, float eps, int H, int G, int KD, int VD, int page_size) {
+    const int* __restrict__ write_slots, T* __restrict__ plane, T* __restrict__ q_out, long ldq, PrepareArgs a, int H, int G,
+    int KD, int VD, int page_size) {
   const long r = blockIdx.x;
   const int u = blockIdx.y, lane = threadIdx.x;
   const long page_stride = (long)G * page_size * (KD + VD);
@@ -31,13 +50,23 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
     const int h = is_q ? u : u - H;
     if (!is_q && !write_slots) return;
     const float* src = proj + r * ldp + (is_q ? q_off : k_off) + (long)h * KD;
-    const float* gain = is_q ? q_gain : k_gain;
-    float ss = 0.f;
-    for (int e = lane; e < KD; e += TIS_WAVE) ss += src[e] * src[e];
-    ss = wave_sum(ss);
-    const float inv = 1.f / sqrtf(ss / (float)KD + eps);
-    const float factor = is_q ? q_factor[h] : 1.f;
-    const float pos = (float)positions[r];
+    const float* bias = is_q ? a.q_bias : a.k_bias;
+    if (bias) bias += (long)h * KD;
+    const float* gain = is_q ? a.q_gain : a.k_gain;
+    float inv = 1.f;
+    if (gain) {
+      float ss = 0.f;
+      for (int e = lane; e < KD; e += TIS_WAVE) {
+        const float v = src[e] + (bias ? bias[e] : 0.f);
+        ss += v * v;
+      }
+      ss = wave_sum(ss);
+      inv = 1.f / sqrtf(ss / (float)KD + a.eps);
+    }
+    float factor = is_q && a.q_factor ? a.q_factor[h] : 1.f;
+    const int ipos = positions[r];
+    if (is_q && a.temp_coef != 0.f) factor *= 1.f + a.temp_coef * logf((float)((ipos + 1) / a.temp_every) + 1.f);
+    const float pos = (float)ipos;
     T* dst;
     if (is_q) {
       dst = q_out + r * ldq + (long)h * KD;
@@ -47,44 +76,104 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
     }
     for (int p = lane; 2 * p < KD; p += TIS_WAVE) {
       const int e0 = 2 * p, e1 = e0 + 1;
-      float a = src[e0] * inv * gain[e0];
-      float b = e1 < KD ? src[e1] * inv * gain[e1] : 0.f;
-      if (e1 < rot_dims) {
+      float x = (src[e0] + (bias ? bias[e0] : 0.f)) * inv * (gain ? gain[e0] : 1.f);
+      float y = e1 < KD ? (src[e1] + (bias ? bias[e1] : 0.f)) * inv * (gain ? gain[e1] : 1.f) : 0.f;
+      if (e1 < a.rot_dims) {
         float sn, cs;
-        sincosf(pos * freqs[p], &sn, &cs);
-        const float ra = a * cs - b * sn, rb = b * cs + a * sn;
-        a = ra;
-        b = rb;
+        sincosf(pos * a.freqs[p], &sn, &cs);
+        const float rx = x * cs - y * sn, ry = y * cs + x * sn;
+        x = rx;
+        y = ry;
       }
-      dst[e0] = from_f<T>(a * factor);
-      if (e1 < KD) dst[e1] = from_f<T>(b * factor);
+      dst[e0] = from_f<T>(x * factor);
+      if (e1 < KD) dst[e1] = from_f<T>(y * factor);
     }
   } else {
     if (!write_slots) return;
     const int h = u - H - G;
     const float* src = proj + r * ldp + v_off + (long)h * VD;
-    float ss = 0.f;
-    for (int e = lane; e < VD; e += TIS_WAVE) ss += src[e] * src[e];
-    ss = wave_sum(ss);
-    const float inv = 1.f / sqrtf(ss / (float)VD + eps);
+    const float* bias = a.v_bias ? a.v_bias + (long)h * VD : nullptr;
+    float inv = 1.f;
+    if (a.value_norm) {
+      float ss = 0.f;
+      for (int e = lane; e < VD; e += TIS_WAVE) {
+        const float v = src[e] + (bias ? bias[e] : 0.f);
+        ss += v * v;
+      }
+      ss = wave_sum(ss);
+      inv = 1.f / sqrtf(ss / (float)VD + a.eps);
+    }
     const int ws = write_slots[r];
     T* dst = plane + (long)(ws / page_size) * page_stride + (long)G * page_size * KD + (long)h * VD * page_size +
              ws % page_size;
-    for (int e = lane; e < VD; e += TIS_WAVE) dst[(long)e * page_size] = from_f<T>(src[e] * inv);
+    for (int e = lane; e < VD; e += TIS_WAVE) dst[(long)e * page_size] = from_f<T>((src[e] + (bias ? bias[e] : 0.f)) * inv);
+  }
+}
+
+// The same step where all heads share one latent as keys and values. grid (rows, H + 1), one wave each.
+// Unit u < H, a query head: the head's R rotated channels (32-bit, at q_off + u * (D + R) + D of proj) are turned by
+// the row's position and written to q_out[u * (C + R) + C ...]; its D unrotated channels go, in the compute type, to
+// q_plain[u * D ...] (for the product that takes them into the latent's space, whose result belongs to
+// q_out[u * (C + R) ...]). Unit H: the row's latent, C channels at c_off, RMS-normed with `gain`, then the R channels
+// of the shared rotated key, turned alike; both go into the row's slot of a page of [slot][C + R] keys.
+template <typename T>
+__global__ __launch_bounds__(TIS_WAVE) void latent_prepare_kernel(
+    const float* __restrict__ proj, long ldp, int q_off, int c_off, const int* __restrict__ positions,
+    const int* __restrict__ write_slots, T* __restrict__ plane, T* __restrict__ q_out, long ldq, T* __restrict__ q_plain,
+    long ldqp, const float* __restrict__ gain, const float* __restrict__ freqs, int rot_dims, float eps, int H, int D,
+    int R, int C, int page_size) {
+  const long r = blockIdx.x;
+  const int u = blockIdx.y, lane = threadIdx.x;
+  const float pos = (float)positions[r];
+  const float* src;
+  T* dst;
+  if (u < H) {
+    src = proj + r * ldp + q_off + (long)u * (D + R);
+    for (int e = lane; e < D; e += TIS_WAVE) q_plain[r * ldqp + (long)u * D + e] = from_f<T>(src[e]);
+    src += D;
+    dst = q_out + r * ldq + (long)u * (C + R) + C;
+  } else {
+    if (!write_slots) return;
+    const int ws = write_slots[r];
+    T* key = plane + ((long)(ws / page_size) * page_size + ws % page_size) * (C + R);
+    src = proj + r * ldp + c_off;
+    float ss = 0.f;
+    for (int e = lane; e < C; e += TIS_WAVE) ss += src[e] * src[e];
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)C + eps);
+    for (int e = lane; e < C; e += TIS_WAVE) key[e] = from_f<T>(src[e] * inv * gain[e]);
+    src += C;
+    dst = key + C;
+  }
+  for (int p = lane; 2 * p < R; p += TIS_WAVE) {
+    const int e0 = 2 * p, e1 = e0 + 1;
+    float x = src[e0], y = e1 < R ? src[e1] : 0.f;
+    if (e1 < rot_dims) {
+      float sn, cs;
+      sincosf(pos * freqs[p], &sn, &cs);
+      const float rx = x * cs - y * sn, ry = y * cs + x * sn;
+      x = rx;
+      y = ry;
+    }
+    dst[e0] = from_f<T>(x);
+    if (e1 < R) dst[e1] = from_f<T>(y);
   }
 }
 
 // One workgroup per (row, query head). Keys are walked in chunks of AW_CHUNK with a running maximum; the order of
-// every sum depends on the row's own position and window only.
+// every sum depends on the row's own position and window only. sink: the softmax's denominator also holds a key of
+// score 0 that has no value. gate (nullable): the head's result is multiplied by sigmoid(gate[row * ldg + head]).
+// latent: a page holds keys only, [slot][KD], and a key's first VD channels are its value.
 template <typename T>
 __global__ __launch_bounds__(AW_THREADS) void attention_window_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ plane, const int* __restrict__ block_tables, int bt_ld,
     const int* __restrict__ row_seq, const int* __restrict__ positions, T* __restrict__ out, long ldo, int group_size,
-    int G, int KD, int VD, int page_size, int window, float scale) {
+    int G, int KD, int VD, int page_size, int window, float scale, int sink, const float* __restrict__ gate, long ldg,
+    int latent) {
   __shared__ float qs[AW_MAX_DIM];
   __shared__ float sc[AW_CHUNK];
   __shared__ float red[16];
-  __shared__ float accm[AW_THREADS];
+  __shared__ float accm[AW_PER][AW_THREADS];
   const long r = blockIdx.x;
   const int h = blockIdx.y, g = h / group_size, t = threadIdx.x;
   const int pos = positions[r];
@@ -93,13 +182,20 @@ __global__ __launch_bounds__(AW_THREADS) void attention_window_kernel(
   const int end = pos + 1;
   for (int d = t; d < KD; d += AW_THREADS) qs[d] = to_f(q[r * ldq + (long)h * KD + d]) * scale;
   __syncthreads();
-  const long page_stride = (long)G * page_size * (KD + VD);
+  const long page_stride = latent ? (long)G * page_size * KD : (long)G * page_size * (KD + VD);
   const long k_off = (long)g * page_size * KD;
-  const long v_off = (long)G * page_size * KD + (long)g * VD * page_size;
-  const int lanes_per_key = AW_THREADS / VD;      // threads that share a value channel, each taking every n-th key
-  const int part = t / VD, d = t % VD;
+  const long v_off = latent ? k_off : (long)G * page_size * KD + (long)g * VD * page_size;
+  const long v_slot = latent ? KD : 1, v_chan = latent ? 1 : page_size;
+  // a thread owns `per` value channels, width apart; the threads that share a channel take every n-th key
+  const int per = (VD + AW_THREADS - 1) / AW_THREADS;
+  const int width = (VD + per - 1) / per;
+  const int lanes_per_key = AW_THREADS / width;
+  const int part = t / width, d = t % width;
   const bool pv = part < lanes_per_key;
-  float m = -INFINITY, l = 0.f, acc = 0.f;
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float acc[AW_PER];
+#pragma unroll
+  for (int u = 0; u < AW_PER; ++u) acc[u] = 0.f;
   for (int c0 = first; c0 < end; c0 += AW_CHUNK) {
     const int n = min(AW_CHUNK, end - c0);
     float cmax = -INFINITY;
@@ -122,65 +218,99 @@ __global__ __launch_bounds__(AW_THREADS) void attention_window_kernel(
     csum = block_sum(csum, red);      // its barriers also publish sc[]
     const float rescale = expf(m - m_new);
     l = l * rescale + csum;
-    acc *= rescale;
+#pragma unroll
+    for (int u = 0; u < AW_PER; ++u) acc[u] *= rescale;
     m = m_new;
     if (pv) {
       for (int i = part; i < n; i += lanes_per_key) {
         const int j = c0 + i;
-        const T* vp = plane + (long)bt[j / page_size] * page_stride + v_off + (j % page_size);
-        acc += sc[i] * to_f(vp[(long)d * page_size]);
+        const T* vp = plane + (long)bt[j / page_size] * page_stride + v_off + (long)(j % page_size) * v_slot;
+        const float p = sc[i];
+#pragma unroll
+        for (int u = 0; u < AW_PER; ++u)
+          if (u < per && d + u * width < VD) acc[u] += p * to_f(vp[(long)(d + u * width) * v_chan]);
       }
     }
     __syncthreads();
   }
-  accm[t] = pv ? acc : 0.f;
+#pragma unroll
+  for (int u = 0; u < AW_PER; ++u) accm[u][t] = pv ? acc[u] : 0.f;
   __syncthreads();
-  if (t < VD) {
+  const float mul = (gate ? 1.f / (1.f + expf(-gate[r * ldg + h])) : 1.f) / l;
+  for (int c = t; c < VD; c += AW_THREADS) {
+    const int u = c / width, dd = c % width;
     float o = 0.f;
-    for (int p = 0; p < lanes_per_key; ++p) o += accm[p * VD + t];
-    out[r * ldo + (long)h * VD + t] = from_f<T>(o / l);
+    for (int p = 0; p < lanes_per_key; ++p) o += accm[u][p * width + dd];
+    out[r * ldo + (long)h * VD + c] = from_f<T>(o * mul);
   }
 }
 
 TIS_EXPORT int tis_attention_prepare(int dtype, const float* proj, long ldp, int q_off, int k_off, int v_off,
                                      const int* positions, const int* write_slots, void* plane, void* q_out, long ldq,
-                                     const float* q_gain, const float* k_gain, const float* q_factor, const float* freqs,
-                                     int rot_dims, float eps, int rows, int H, int G, int KD, int VD, int page_size,
-                                     hipStream_t stream) {
+                                     const float* q_bias, const float* k_bias, const float* v_bias, const float* q_gain,
+                                     const float* k_gain, const float* q_factor, const float* freqs, int rot_dims, float eps,
+                                     int value_norm, float temp_coef, int temp_every, int rows, int H, int G, int KD, int VD,
+                                     int page_size, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || H < 1 || G < 1 || KD < 1 || VD < 1 || page_size < 1 || H + 2 * G > 65535)
     return tis_fail("attention_prepare: bad size rows=%d heads=%d kv_heads=%d key=%d value=%d page=%d", rows, H, G, KD, VD,
                     page_size);
-  if (rot_dims < 0 || rot_dims > KD || rot_dims % 2) return tis_fail("attention_prepare: %d rotated channels of %d", rot_dims, KD);
+  if (rot_dims < 0 || rot_dims > KD || rot_dims % 2 || (rot_dims && !freqs))
+    return tis_fail("attention_prepare: %d rotated channels of %d", rot_dims, KD);
+  if (temp_coef != 0.f && temp_every < 1) return tis_fail("attention_prepare: a query factor every %d positions", temp_every);
   if (write_slots && !plane) return tis_fail("attention_prepare: write slots without pages");
+  PrepareArgs a{q_bias, k_bias, v_bias, q_gain, k_gain, q_factor, freqs, rot_dims, eps, value_norm, temp_coef, temp_every};
   dim3 grid(rows, H + 2 * G);
   if (dtype == TIS_F32)
     attention_prepare_kernel<float><<<grid, TIS_WAVE, 0, stream>>>(proj, ldp, q_off, k_off, v_off, positions, write_slots,
-        (float*)plane, (float*)q_out, ldq, q_gain, k_gain, q_factor, freqs, rot_dims, eps, H, G, KD, VD, page_size);
+        (float*)plane, (float*)q_out, ldq, a, H, G, KD, VD, page_size);
   else if (dtype == TIS_BF16)
     attention_prepare_kernel<bf16><<<grid, TIS_WAVE, 0, stream>>>(proj, ldp, q_off, k_off, v_off, positions, write_slots,
-        (bf16*)plane, (bf16*)q_out, ldq, q_gain, k_gain, q_factor, freqs, rot_dims, eps, H, G, KD, VD, page_size);
+        (bf16*)plane, (bf16*)q_out, ldq, a, H, G, KD, VD, page_size);
   else
     return tis_fail("unknown dtype code %d", dtype);
   return tis_launch_status("attention_prepare");
 }
 
+TIS_EXPORT int tis_latent_prepare(int dtype, const float* proj, long ldp, int q_off, int c_off, const int* positions,
+                                  const int* write_slots, void* plane, void* q_out, long ldq, void* q_plain, long ldqp,
+                                  const float* gain, const float* freqs, int rot_dims, float eps, int rows, int H, int D,
+                                  int R, int C, int page_size, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || H < 1 || H > 65534 || D < 0 || R < 0 || C < 1 || page_size < 1 || !gain || !q_out || (D && !q_plain))
+    return tis_fail("latent_prepare: bad size rows=%d heads=%d dim=%d rotated=%d latent=%d page=%d", rows, H, D, R, C, page_size);
+  if (rot_dims < 0 || rot_dims > R || rot_dims % 2 || (rot_dims && !freqs))
+    return tis_fail("latent_prepare: %d rotated channels of %d", rot_dims, R);
+  if (write_slots && !plane) return tis_fail("latent_prepare: write slots without pages");
+  dim3 grid(rows, H + 1);
+  if (dtype == TIS_F32)
+    latent_prepare_kernel<float><<<grid, TIS_WAVE, 0, stream>>>(proj, ldp, q_off, c_off, positions, write_slots, (float*)plane,
+        (float*)q_out, ldq, (float*)q_plain, ldqp, gain, freqs, rot_dims, eps, H, D, R, C, page_size);
+  else if (dtype == TIS_BF16)
+    latent_prepare_kernel<bf16><<<grid, TIS_WAVE, 0, stream>>>(proj, ldp, q_off, c_off, positions, write_slots, (bf16*)plane,
+        (bf16*)q_out, ldq, (bf16*)q_plain, ldqp, gain, freqs, rot_dims, eps, H, D, R, C, page_size);
+  else
+    return tis_fail("unknown dtype code %d", dtype);
+  return tis_launch_status("latent_prepare");
+}
+
 TIS_EXPORT int tis_attention_window(int dtype, const void* q, long ldq, const void* plane, const int* block_tables,
                                     int bt_ld, const int* row_seq, const int* positions, void* out, long ldo, int rows,
-                                    int H, int G, int KD, int VD, int page_size, int window, float scale,
-                                    hipStream_t stream) {
+                                    int H, int G, int KD, int VD, int page_size, int window, float scale, int sink,
+                                    const float* gate, long ldg, int latent, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || H < 1 || G < 1 || H % G || page_size < 1 || window < 0 || H > 65535)
     return tis_fail("attention_window: bad size rows=%d heads=%d kv_heads=%d page=%d window=%d", rows, H, G, page_size, window);
   if (KD < 1 || KD > AW_MAX_DIM || VD < 1 || VD > AW_MAX_DIM)
     return tis_fail("attention_window: key size %d or value size %d is outside 1..%d", KD, VD, AW_MAX_DIM);
+  if (latent && VD > KD) return tis_fail("attention_window: a latent's value (%d) is part of its key (%d)", VD, KD);
   dim3 grid(rows, H);
   if (dtype == TIS_F32)
     attention_window_kernel<float><<<grid, AW_THREADS, 0, stream>>>((const float*)q, ldq, (const float*)plane, block_tables,
-        bt_ld, row_seq, positions, (float*)out, ldo, H / G, G, KD, VD, page_size, window, scale);
+        bt_ld, row_seq, positions, (float*)out, ldo, H / G, G, KD, VD, page_size, window, scale, sink, gate, ldg, latent);
   else if (dtype == TIS_BF16)
     attention_window_kernel<bf16><<<grid, AW_THREADS, 0, stream>>>((const bf16*)q, ldq, (const bf16*)plane, block_tables,
-        bt_ld, row_seq, positions, (bf16*)out, ldo, H / G, G, KD, VD, page_size, window, scale);
+        bt_ld, row_seq, positions, (bf16*)out, ldo, H / G, G, KD, VD, page_size, window, scale, sink, gate, ldg, latent);
   else
     return tis_fail("unknown dtype code %d", dtype);
   return tis_launch_status("attention_window");

@@ -1,0 +1,274 @@
+// Routed feed-forwards (mixtures of experts) and other products that come in groups: the router's choice, the lists of
+// rows per expert, a grouped product C_g = act(A_g . W_g^T), and the weighted sum of a row's chosen experts.
+//
+// Router: s = softmax(z) over all of a row's router outputs in 32-bit; the `top` outputs with the largest s + correction
+// are chosen (the lower index wins a tie); a chosen output's weight is s * scale, taken without the correction and not
+// renormalised. Outputs from n_experts on are identity experts: they have no matrices, their result is the row itself.
+//
+// An assignment is a (row, k-th choice) pair, numbered row * top + k. The lists kernel gives every expert the
+// assignments that chose it, in rising order, in a line of `rows` entries of its own (an expert is chosen at most once
+// a row), so nothing needs a prefix sum or an atomic and the order never depends on timing.
+//
+// The grouped product walks, for group g, tiles of 16 list entries against tiles of 64 output columns of the group's
+// matrix W[g] ([N][K]). Entry e's input row is A + (e / a_div) * lda + g * a_group, its output row C + e * ldc +
+// g * c_group: with a_div = top the input rows are the step's rows and the outputs lie by assignment (an expert's first
+// product), with a_div = 1 both lie by assignment (its second); without lists every group takes all rows, and a_group /
+// c_group move from one group's columns to the next (a product per head on a head's own columns). Sums are 32-bit in
+// an order that depends on K alone, so a row's result does not depend on what else is in the step.
+#include "common.h"
+
+TIS_DEFINE_LAST_ERROR(tis_experts)
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+static constexpr int EX_MAX_PER_LANE = 16;      // router outputs a lane keeps: up to 1,024 outputs a row
+
+__device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.f + erff(z * 0.7071067811865476f)); }
+
+// one wave per row
+__global__ __launch_bounds__(TIS_WAVE) void route_topk_kernel(const float* __restrict__ z, long ldz,
+                                                              const float* __restrict__ correction, float scale,
+                                                              int n_out, int top, int* __restrict__ ids,
+                                                              float* __restrict__ weights) {
+  const long r = blockIdx.x;
+  const int lane = threadIdx.x;
+  float s[EX_MAX_PER_LANE], c[EX_MAX_PER_LANE];
+  float m = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
+    const int e = lane + u * TIS_WAVE;
+    s[u] = e < n_out ? z[r * ldz + e] : -INFINITY;
+    m = fmaxf(m, s[u]);
+  }
+  m = wave_max(m);
+  float sum = 0.f;
+#pragma unroll
+  for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
+    const int e = lane + u * TIS_WAVE;
+    s[u] = e < n_out ? expf(s[u] - m) : 0.f;
+    sum += s[u];
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.f / sum;
+#pragma unroll
+  for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
+    const int e = lane + u * TIS_WAVE;
+    s[u] *= inv;
+    c[u] = e < n_out ? s[u] + (correction ? correction[e] : 0.f) : -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
+      const int e = lane + u * TIS_WAVE;
+      if (c[u] > best) { best = c[u]; at = e; }       // rising e within a lane: the lower index keeps a tie
+    }
+#pragma unroll
+    for (int o = TIS_WAVE / 2; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, TIS_WAVE);
+      const int oa = __shfl_xor(at, o, TIS_WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    float w = 0.f;
+#pragma unroll
+    for (int u = 0; u < EX_MAX_PER_LANE; ++u) {
+      if (lane + u * TIS_WAVE == at) { w = s[u]; c[u] = -INFINITY; }
+    }
+    w = wave_sum(w);          // only the owner's lane holds it
+    if (lane == 0) {
+      ids[r * top + k] = at;
+      weights[r * top + k] = w * scale;
+    }
+  }
+}
+
+// one workgroup per expert: the assignments that chose it, in rising order
+__global__ __launch_bounds__(256) void expert_lists_kernel(const int* __restrict__ ids, int n_assign, int line,
+                                                           int* __restrict__ lists, int* __restrict__ counts) {
+  __shared__ int wave_count[4];
+  __shared__ int base;
+  const int e = blockIdx.x, t = threadIdx.x, lane = t % TIS_WAVE, wave = t / TIS_WAVE;
+  if (t == 0) base = 0;
+  __syncthreads();
+  for (int a0 = 0; a0 < n_assign; a0 += 256) {
+    const int a = a0 + t;
+    const bool mine = a < n_assign && ids[a] == e;
+    const unsigned long long vote = __ballot(mine);
+    const int before = __popcll(vote & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_count[wave] = __popcll(vote);
+    __syncthreads();
+    int off = base;
+    for (int w = 0; w < wave; ++w) off += wave_count[w];
+    if (mine) lists[(long)e * line + off + before] = a;
+    __syncthreads();
+    if (t == 0) base += wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+    __syncthreads();
+  }
+  if (t == 0) counts[e] = base;
+}
+
+struct GroupedArgs {
+  const int* lists;     // [groups][line] entries, or null: every group takes the entries 0 .. rows-1
+  const int* counts;    // [groups], with lists
+  int line, rows, a_div;
+  long lda, a_group, ldc, c_group;
+  int N, K, act;        // act 0: none, 1: erf-form gelu
+};
+
+// plain multiply-adds, any type and any alignment: 16 entries x 64 columns a workgroup, K in steps of 32 through LDS
+template <typename TA, typename TO>
+__global__ __launch_bounds__(256) void grouped_plain_kernel(const TA* __restrict__ A, const TA* __restrict__ W,
+                                                            TO* __restrict__ C, GroupedArgs p) {
+  __shared__ float As[16][33];
+  __shared__ float Ws[64][33];
+  __shared__ int entry[16];
+  const int g = blockIdx.z, m0 = blockIdx.y * 16, n0 = blockIdx.x * 64, t = threadIdx.x;
+  const int count = p.lists ? p.counts[g] : p.rows;
+  if (m0 >= count) return;
+  if (t < 16) entry[t] = m0 + t < count ? (p.lists ? p.lists[(long)g * p.line + m0 + t] : m0 + t) : -1;
+  __syncthreads();
+  const TA* Wg = W + (long)g * p.N * p.K;
+  const int tx = t % 64, ty = t / 64;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < p.K; k0 += 32) {
+    for (int i = t; i < 16 * 32; i += 256) {
+      const int row = i / 32, kk = i % 32, e = entry[row];
+      As[row][kk] = (e >= 0 && k0 + kk < p.K) ? to_f(A[(long)(e / p.a_div) * p.lda + (long)g * p.a_group + k0 + kk]) : 0.f;
+    }
+    for (int i = t; i < 64 * 32; i += 256) {
+      const int col = i / 32, kk = i % 32;
+      Ws[col][kk] = (n0 + col < p.N && k0 + kk < p.K) ? to_f(Wg[(long)(n0 + col) * p.K + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 32; ++kk) {
+      const float w = Ws[tx][kk];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] += As[ty * 4 + i][kk] * w;
+    }
+    __syncthreads();
+  }
+  if (n0 + tx >= p.N) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int e = entry[ty * 4 + i];
+    if (e < 0) continue;
+    const float v = p.act == 1 ? gelu_erf_f(acc[i]) : acc[i];
+    C[(long)e * p.ldc + (long)g * p.c_group + n0 + tx] = from_f<TO>(v);
+  }
+}
+
+// bfloat16 on the matrix cores: a wave owns 16 entries x 16 columns, four waves a workgroup side by side in N. A
+// matrix row and an input row are the two operands of v_mfma_f32_16x16x32_bf16 straight from memory, 16 bytes a lane
+// (rows 16-byte aligned, K a multiple of 8). Each result is one wave's sum over K in steps of 32.
+template <typename TO>
+__global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                           TO* __restrict__ C, GroupedArgs p) {
+  const int g = blockIdx.z, m0 = blockIdx.y * 16, t = threadIdx.x, lane = t % 64, wave = t / 64;
+  const int n0 = blockIdx.x * 64 + wave * 16;
+  const int count = p.lists ? p.counts[g] : p.rows;
+  if (m0 >= count || n0 >= p.N) return;
+  const int c16 = lane & 15, kg = lane >> 4;
+  const int mine = m0 + c16 < count ? (p.lists ? p.lists[(long)g * p.line + m0 + c16] : m0 + c16) : -1;
+  const bf16* arow = A + (long)(mine < 0 ? 0 : mine / p.a_div) * p.lda + (long)g * p.a_group + kg * 8;
+  const bool w_ok = n0 + c16 < p.N;
+  const bf16* wrow = W + ((long)g * p.N + (w_ok ? n0 + c16 : 0)) * p.K + kg * 8;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < p.K; k0 += 32) {
+    const bool k_ok = k0 + kg * 8 < p.K;
+    const bf16x8 wv = (w_ok && k_ok) ? *reinterpret_cast<const bf16x8*>(wrow + k0) : zero;
+    const bf16x8 av = (mine >= 0 && k_ok) ? *reinterpret_cast<const bf16x8*>(arow + k0) : zero;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc, 0, 0, 0);
+  }
+  // the lane holds the columns n0 + 4 kg + i of entry c16
+  if (mine < 0) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = n0 + 4 * kg + i;
+    if (n >= p.N) continue;
+    const float v = p.act == 1 ? gelu_erf_f(acc[i]) : acc[i];
+    C[(long)mine * p.ldc + (long)g * p.c_group + n] = from_f<TO>(v);
+  }
+}
+
+// out[r] = sum_k weight[r][k] * (y[r * top + k] if ids[r][k] < n_experts else x[r]), in 32-bit
+template <typename T>
+__global__ __launch_bounds__(256) void experts_combine_kernel(const float* __restrict__ y, long ldy, const T* __restrict__ x,
+                                                              long ldx, const int* __restrict__ ids,
+                                                              const float* __restrict__ weights, int top, int n_experts,
+                                                              float* __restrict__ out, long ldo, int D) {
+  const long r = blockIdx.x;
+  for (int c = threadIdx.x; c < D; c += 256) {
+    float v = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int e = ids[r * top + k];
+      const float w = weights[r * top + k];
+      v += w * (e < n_experts ? y[(r * top + k) * ldy + c] : to_f(x[r * ldx + c]));
+    }
+    out[r * ldo + c] = v;
+  }
+}
+
+TIS_EXPORT int tis_route_topk(const float* z, long ldz, const float* correction, float scale, int rows, int n_out, int top,
+                              int* ids, float* weights, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || n_out < 1 || n_out > EX_MAX_PER_LANE * TIS_WAVE || top < 1 || top > n_out)
+    return tis_fail("route_topk: bad size rows=%d outputs=%d (at most %d) top=%d", rows, n_out, EX_MAX_PER_LANE * TIS_WAVE, top);
+  route_topk_kernel<<<rows, TIS_WAVE, 0, stream>>>(z, ldz, correction, scale, n_out, top, ids, weights);
+  return tis_launch_status("route_topk");
+}
+
+TIS_EXPORT int tis_expert_lists(const int* ids, int n_assign, int n_experts, int line, int* lists, int* counts,
+                                hipStream_t stream) {
+  if (n_experts == 0) return 0;
+  if (n_assign < 0 || n_experts < 0 || line < 1) return tis_fail("expert_lists: bad size assignments=%d experts=%d", n_assign, n_experts);
+  expert_lists_kernel<<<n_experts, 256, 0, stream>>>(ids, n_assign, line, lists, counts);
+  return tis_launch_status("expert_lists");
+}
+
+// in_dtype / out_dtype: 0 float, 1 bfloat16 (a bfloat16 input may give a 32-bit output). most_rows: the most entries a
+// group can have (the grid's height).
+TIS_EXPORT int tis_grouped_linear(int in_dtype, int out_dtype, const void* A, long lda, long a_group, int a_div, const void* W,
+                                  void* C, long ldc, long c_group, const int* lists, const int* counts, int line,
+                                  int groups, int most_rows, int N, int K, int act, hipStream_t stream) {
+  if (groups == 0 || most_rows == 0) return 0;
+  if (groups < 0 || groups > 65535 || most_rows < 0 || N < 1 || K < 1 || a_div < 1 || (act != 0 && act != 1))
+    return tis_fail("grouped_linear: bad size groups=%d rows=%d N=%d K=%d", groups, most_rows, N, K);
+  if ((lists == nullptr) != (counts == nullptr)) return tis_fail("grouped_linear: lists and counts go together");
+  const int tiles_m = (most_rows + 15) / 16;
+  if (tiles_m > 65535) return tis_fail("grouped_linear: %d rows are too many for one call", most_rows);
+  GroupedArgs p{lists, counts, line, most_rows, a_div, lda, a_group, ldc, c_group, N, K, act};
+  dim3 grid((N + 63) / 64, tiles_m, groups);
+  if (in_dtype == TIS_BF16) {
+    const bool aligned = K % 8 == 0 && lda % 8 == 0 && a_group % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0;
+    if (aligned) {
+      if (out_dtype == TIS_BF16) grouped_mfma_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (bf16*)C, p);
+      else grouped_mfma_kernel<float><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (float*)C, p);
+    } else {
+      if (out_dtype == TIS_BF16) grouped_plain_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (bf16*)C, p);
+      else grouped_plain_kernel<bf16, float><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (float*)C, p);
+    }
+  } else if (in_dtype == TIS_F32 && out_dtype == TIS_F32) {
+    grouped_plain_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)A, (const float*)W, (float*)C, p);
+  } else {
+    return tis_fail("grouped_linear: dtype codes %d -> %d", in_dtype, out_dtype);
+  }
+  return tis_launch_status("grouped_linear");
+}
+
+TIS_EXPORT int tis_experts_combine(int dtype, const float* y, long ldy, const void* x, long ldx, const int* ids,
+                                   const float* weights, int top, int n_experts, float* out, long ldo, int rows, int D,
+                                   hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1 || top < 1) return tis_fail("experts_combine: bad size rows=%d width=%d top=%d", rows, D, top);
+  if (dtype == TIS_F32)
+    experts_combine_kernel<float><<<rows, 256, 0, stream>>>(y, ldy, (const float*)x, ldx, ids, weights, top, n_experts, out, ldo, D);
+  else if (dtype == TIS_BF16)
+    experts_combine_kernel<bf16><<<rows, 256, 0, stream>>>(y, ldy, (const bf16*)x, ldx, ids, weights, top, n_experts, out, ldo, D);
+  else
+    return tis_fail("unknown dtype code %d", dtype);
+  return tis_launch_status("experts_combine");
+}

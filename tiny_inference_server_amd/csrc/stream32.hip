@@ -135,6 +135,103 @@ __global__ __launch_bounds__(S32_THREADS) void lowrank_decay_kernel(const float*
   }
 }
 
+
+// Layer norm of a 32-bit row into the compute type: (x - mean) / sqrt(var + eps) * gain + bias, the variance being the
+// mean of the squared deviations (two passes over the row; bias may be null).
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void layernorm32_kernel(const float* __restrict__ x, const float* __restrict__ gain,
+                                                                   const float* __restrict__ bias, float eps,
+                                                                   T* __restrict__ out, long ldo, int D) {
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) s += x[r * D + c];
+  const float mean = block_sum(s, red) / (float)D;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    const float d = x[r * D + c] - mean;
+    ss += d * d;
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)D + eps);
+  for (int c = threadIdx.x; c < D; c += S32_THREADS)
+    out[r * ldo + c] = from_f<T>((x[r * D + c] - mean) * inv * gain[c] + (bias ? bias[c] : 0.f));
+}
+
+// The residual sum of a 32-bit stream, with what usually follows it, in one pass over the row:
+//   v = x + y                                  (y_gain null)
+//   v = x + y / sqrt(mean(y^2) + y_eps) * y_gain   (an RMS norm on the branch before the sum)
+// v goes to out32 (which may be x itself); `copy` (nullable) gets v in the compute type; `normed` (nullable) gets the
+// norm of v in the compute type: kind 1 layer norm (gain, bias), kind 2 RMS norm (gain), eps under the root in both.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
+    const float* __restrict__ x, const float* __restrict__ y, long ldy, const float* __restrict__ y_gain, float y_eps,
+    float* __restrict__ out32, T* __restrict__ copy, long ldc, int norm_kind, const float* __restrict__ gain,
+    const float* __restrict__ bias, float eps, T* __restrict__ normed, long ldn, int D) {
+  __shared__ float red[16];
+  const long r = blockIdx.x;
+  float y_inv = 1.f;
+  if (y && y_gain) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+      const float v = y[r * ldy + c];
+      ss += v * v;
+    }
+    y_inv = 1.f / sqrtf(block_sum(ss, red) / (float)D + y_eps);
+  }
+  float s = 0.f;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    float v = x[r * D + c];
+    if (y) v += y_gain ? y[r * ldy + c] * y_inv * y_gain[c] : y[r * ldy + c];
+    out32[r * D + c] = v;          // (each thread reads back only what it wrote itself)
+    if (copy) copy[r * ldc + c] = from_f<T>(v);
+    s += norm_kind == 2 ? v * v : v;
+  }
+  if (!normed || norm_kind == 0) return;
+  if (norm_kind == 2) {
+    const float inv = 1.f / sqrtf(block_sum(s, red) / (float)D + eps);
+    for (int c = threadIdx.x; c < D; c += S32_THREADS) normed[r * ldn + c] = from_f<T>(out32[r * D + c] * inv * gain[c]);
+    return;
+  }
+  const float mean = block_sum(s, red) / (float)D;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+    const float d = out32[r * D + c] - mean;
+    ss += d * d;
+  }
+  const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)D + eps);
+  for (int c = threadIdx.x; c < D; c += S32_THREADS)
+    normed[r * ldn + c] = from_f<T>((out32[r * D + c] - mean) * inv * gain[c] + (bias ? bias[c] : 0.f));
+}
+
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// out[r][j] = act(z[r][j]) * table[token[r]][j]: a gate on a row of a per-token table. act 0: tanh-form gelu, 1: silu,
+// 2: sigmoid. z is 32-bit (a strided view is fine), table and out are in the compute type.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void gate_table_kernel(const float* __restrict__ z, long ldz,
+                                                                  const T* __restrict__ table, long ldt,
+                                                                  const int* __restrict__ tokens, int act,
+                                                                  T* __restrict__ out, long ldo, int rows, int W) {
+  const long i = (long)blockIdx.x * S32_THREADS + threadIdx.x;
+  if (i >= (long)rows * W) return;
+  const long r = i / W;
+  const int j = (int)(i % W);
+  const float v = z[r * ldz + j];
+  const float a = act == 0 ? gelu_tanh_f(v) : act == 1 ? v * sigmoid_f(v) : sigmoid_f(v);
+  out[r * ldo + j] = from_f<T>(a * to_f(table[(long)tokens[r] * ldt + j]));
+}
+
+// In place on the columns [0, W) of 32-bit rows: act 1 silu, 2 sigmoid, 0 tanh-form gelu.
+__global__ __launch_bounds__(S32_THREADS) void activate32_kernel(float* __restrict__ z, long ldz, int act, int rows, int W) {
+  const long i = (long)blockIdx.x * S32_THREADS + threadIdx.x;
+  if (i >= (long)rows * W) return;
+  float* p = z + (i / W) * ldz + (i % W);
+  const float v = *p;
+  *p = act == 0 ? gelu_tanh_f(v) : act == 1 ? v * sigmoid_f(v) : sigmoid_f(v);
+}
+
 #define S32_DISPATCH(call_f32, call_bf16)                 \
   if (dtype == TIS_F32) { call_f32; }                     \
   else if (dtype == TIS_BF16) { call_bf16; }              \
@@ -195,4 +292,45 @@ TIS_EXPORT int tis_lowrank_decay(const float* low, long ldl, int rank, const flo
     return tis_fail("lowrank_decay: bad size rows=%d rank=%d channels=%d tau=%g", rows, rank, C, (double)tau);
   lowrank_decay_kernel<<<rows, S32_THREADS, rank * sizeof(float), stream>>>(low, ldl, rank, w2, bias, tau, out, C);
   return tis_launch_status("lowrank_decay");
+}
+
+TIS_EXPORT int tis_layernorm32(int dtype, const float* x, const float* gain, const float* bias, float eps, void* out, long ldo,
+                               int rows, int D, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1 || !x || !gain || !out) return tis_fail("layernorm32: bad arguments rows=%d width=%d", rows, D);
+  S32_DISPATCH((layernorm32_kernel<float><<<rows, S32_THREADS, 0, stream>>>(x, gain, bias, eps, (float*)out, ldo, D)),
+               (layernorm32_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>(x, gain, bias, eps, (bf16*)out, ldo, D)))
+  return tis_launch_status("layernorm32");
+}
+
+TIS_EXPORT int tis_residual_norm(int dtype, const float* x, const float* y, long ldy, const float* y_gain, float y_eps,
+                                 float* out32, void* copy, long ldc, int norm_kind, const float* gain, const float* bias,
+                                 float eps, void* normed, long ldn, int rows, int D, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || D < 1 || !x || !out32) return tis_fail("residual_norm: bad arguments rows=%d width=%d", rows, D);
+  if (norm_kind < 0 || norm_kind > 2 || (norm_kind && (!gain || !normed)))
+    return tis_fail("residual_norm: norm kind %d needs a gain and an output", norm_kind);
+  S32_DISPATCH((residual_norm_kernel<float><<<rows, S32_THREADS, 0, stream>>>(x, y, ldy, y_gain, y_eps, out32, (float*)copy, ldc,
+                                                                             norm_kind, gain, bias, eps, (float*)normed, ldn, D)),
+               (residual_norm_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>(x, y, ldy, y_gain, y_eps, out32, (bf16*)copy, ldc,
+                                                                            norm_kind, gain, bias, eps, (bf16*)normed, ldn, D)))
+  return tis_launch_status("residual_norm");
+}
+
+TIS_EXPORT int tis_gate_table(int dtype, const float* z, long ldz, const void* table, long ldt, const int* tokens, int act,
+                              void* out, long ldo, int rows, int W, hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || W < 1 || act < 0 || act > 2) return tis_fail("gate_table: bad size rows=%d width=%d act=%d", rows, W, act);
+  const long blocks = ((long)rows * W + S32_THREADS - 1) / S32_THREADS;
+  S32_DISPATCH((gate_table_kernel<float><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, (const float*)table, ldt, tokens, act, (float*)out, ldo, rows, W)),
+               (gate_table_kernel<bf16><<<blocks, S32_THREADS, 0, stream>>>(z, ldz, (const bf16*)table, ldt, tokens, act, (bf16*)out, ldo, rows, W)))
+  return tis_launch_status("gate_table");
+}
+
+TIS_EXPORT int tis_activate32(float* z, long ldz, int act, int rows, int W, hipStream_t stream) {
+  if (rows == 0 || W == 0) return 0;
+  if (rows < 0 || W < 0 || act < 0 || act > 2) return tis_fail("activate32: bad size rows=%d width=%d act=%d", rows, W, act);
+  const long blocks = ((long)rows * W + S32_THREADS - 1) / S32_THREADS;
+  activate32_kernel<<<blocks, S32_THREADS, 0, stream>>>(z, ldz, act, rows, W);
+  return tis_launch_status("activate32");
 }

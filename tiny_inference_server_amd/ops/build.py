@@ -43,6 +43,7 @@ SOURCES: Dict[str, str] = {
     "stream32": "stream32.hip",
     "attention_window": "attention_window.hip",
     "state_scan": "state_scan.hip",
+    "experts": "experts.hip",
 }
 HEADERS = ["common.h", "attention_mfma.h"]
 # what a library links beyond the HIP runtime

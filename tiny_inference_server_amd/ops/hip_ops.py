@@ -107,10 +107,22 @@ _SIGNATURES["stream32"] = ("tis_stream32", {
     "tis_rmsnorm32": [_I, _P, _P, _F, _P, _L, _I, _I, _P],
     "tis_head_norm_gate": [_I, _P, _L, _P, _L, _P, _I, _I, _F, _P, _L, _I, _I, _I, _P],
     "tis_lowrank_decay": [_P, _L, _I, _P, _P, _F, _P, _I, _I, _P],
+    "tis_layernorm32": [_I, _P, _P, _P, _F, _P, _L, _I, _I, _P],
+    "tis_residual_norm": [_I, _P, _P, _L, _P, _F, _P, _P, _L, _I, _P, _P, _F, _P, _L, _I, _I, _P],
+    "tis_gate_table": [_I, _P, _L, _P, _L, _P, _I, _P, _L, _I, _I, _P],
+    "tis_activate32": [_P, _L, _I, _I, _I, _P],
 })
 _SIGNATURES["attention_window"] = ("tis_attention_window", {
-    "tis_attention_prepare": [_I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P],
-    "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+    "tis_attention_prepare": [_I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _F, _I,
+                              _I, _I, _I, _I, _I, _I, _P],
+    "tis_latent_prepare": [_I, _P, _L, _I, _I, _P, _P, _P, _P, _L, _P, _L, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P],
+    "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _I, _P],
+})
+_SIGNATURES["experts"] = ("tis_experts", {
+    "tis_route_topk": [_P, _L, _P, _F, _I, _I, _I, _P, _P, _P],
+    "tis_expert_lists": [_P, _I, _I, _I, _P, _P, _P],
+    "tis_grouped_linear": [_I, _I, _P, _L, _L, _I, _P, _P, _L, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "tis_experts_combine": [_I, _P, _L, _P, _L, _P, _P, _I, _I, _P, _L, _I, _I, _P],
 })
 _SIGNATURES["state_scan"] = ("tis_state_scan", {
     "tis_state_scan": [_I, _P, _L, _I, _I, _I, _F, _P, _L, _I, _I, _P, _P, _F, _P, _L, _P, _P, _I, _P, _L, _I, _I, _I, _I,
@@ -1121,6 +1133,143 @@ class HipOps:
                                                  _ptr(out), n, C, self._stream())
         return out
 
+    def layernorm32(self, x32, gain, bias, eps: float):
+        """(x - mean) / sqrt(var + eps) * gain + bias of 32-bit rows, in the compute type (bias may be None)."""
+        n, D = x32.shape
+        self._f32(x32, "layernorm32 x", n * D)
+        self._f32(gain, "layernorm32 gain", D)
+        if bias is not None:
+            self._f32(bias, "layernorm32 bias", D)
+        out = self.empty(n, D)
+        self._lazy("stream32").tis_layernorm32(self.code, _ptr(x32), _ptr(gain), _ptr(bias), float(eps), _ptr(out),
+                                               out.stride(0), n, D, self._stream())
+        return out
+
+    def residual_norm(self, x32, y=None, y_rms=None, copy=False, norm=None):
+        """x32 <- x32 + y, in place, with what usually follows: (x32, copy, normed).
+
+        y: [rows, width] 32-bit (a strided view is fine) or None; y_rms = (gain, eps): y is RMS-normed with that gain
+        before it is added. copy: also return the new rows in the compute type. norm = (kind, gain, bias, eps) with kind
+        "layer" (bias may be None) or "rms": also return the norm of the new rows in the compute type. In a 32-bit
+        engine the copy is the stream itself."""
+        n, D = x32.shape
+        self._f32(x32, "residual_norm x", n * D)
+        if y is not None:
+            self._f32_rows(y, "residual_norm y", n, D)
+        elif y_rms is not None:
+            raise KernelError("residual_norm: a norm on a branch that is not there")
+        if y_rms is not None:
+            self._f32(y_rms[0], "residual_norm branch gain", D)
+        kind, gain, bias, eps = 0, None, None, 0.0
+        if norm is not None:
+            kind = {"layer": 1, "rms": 2}[norm[0]]
+            gain, bias, eps = norm[1], norm[2], norm[3]
+            self._f32(gain, "residual_norm gain", D)
+            if bias is not None:
+                self._f32(bias, "residual_norm bias", D)
+        as_is = self.dtype == torch.float32
+        cp = self.empty(n, D) if copy and not as_is else None
+        normed = self.empty(n, D) if kind else None
+        self._lazy("stream32").tis_residual_norm(
+            self.code, _ptr(x32), _ptr(y), y.stride(0) if y is not None else 0, _ptr(y_rms[0] if y_rms else None),
+            float(y_rms[1]) if y_rms else 0.0, _ptr(x32), _ptr(cp), cp.stride(0) if cp is not None else 0, kind, _ptr(gain),
+            _ptr(bias), float(eps), _ptr(normed), normed.stride(0) if normed is not None else 0, n, D, self._stream())
+        return x32, (x32 if copy and as_is else cp), normed
+
+    _ACTS = {"gelu_tanh": 0, "silu": 1, "sigmoid": 2}
+
+    def gate_table(self, z, table, tokens, act: str):
+        """act(z) * table[tokens]: z [rows, W] 32-bit (a strided view is fine), table [entries, W] in the compute type;
+        the result [rows, W] in the compute type. act: "gelu_tanh", "silu" or "sigmoid"."""
+        n, W = z.shape
+        self._f32_rows(z, "gate_table z", n, W)
+        _rows_view(self._check(table, "gate_table table"), "gate_table table")
+        if table.shape[1] != W:
+            raise KernelError(f"gate_table: table rows of {table.shape[1]} for gates of {W}")
+        self._index(tokens, "tokens", n)
+        out = self.empty(n, W)
+        self._lazy("stream32").tis_gate_table(self.code, _ptr(z), z.stride(0), _ptr(table), table.stride(0), _ptr(tokens),
+                                              self._ACTS[act], _ptr(out), out.stride(0), n, W, self._stream())
+        return out
+
+    def activate32(self, z, act: str):
+        """act on 32-bit rows, in place (z may be a strided view of some columns)."""
+        _rows_view(self._check(z, "activate32 z", torch.float32), "activate32 z")
+        self._lazy("stream32").tis_activate32(_ptr(z), z.stride(0), self._ACTS[act], z.shape[0], z.shape[1], self._stream())
+        return z
+
+    # ---- products in groups: experts, heads -----------------------------------------------------------------
+    def _grouped(self, a, lda, a_group, a_div, w, c, ldc, c_group, lists, counts, line, most_rows, act=0):
+        G, N, K = w.shape
+        self._check(w, "grouped product matrices")
+        if not w.is_contiguous():
+            raise KernelError("grouped product: the matrices must be contiguous [groups, out, in]")
+        self._lazy("experts").tis_grouped_linear(
+            _DT[a.dtype], _DT[c.dtype], _ptr(a), lda, a_group, a_div, _ptr(w), _ptr(c), ldc, c_group, _ptr(lists),
+            _ptr(counts), line, G, most_rows, N, K, act, self._stream())
+
+    def heads_linear(self, x, w, out, out_group: int, out_offset: int = 0):
+        """A product per head on the head's own columns: out[:, out_offset + h * out_group + (0..N)] =
+        x[:, h * K + (0..K)] . w[h]^T for w [heads, N, K]. x: [rows, heads * K] in the compute type; out: a 2-d tensor
+        of the compute type or 32-bit whose other columns are left as they are."""
+        _rows_view(self._check(x, "heads_linear x"), "heads_linear x")
+        H, N, K = w.shape
+        n = x.shape[0]
+        if x.shape[1] != H * K:
+            raise KernelError(f"heads_linear: x has {x.shape[1]} columns for {H} heads of {K}")
+        if out.dtype not in (self.dtype, torch.float32):
+            raise KernelError(f"heads_linear: out dtype {out.dtype}")
+        _rows_view(self._check(out, "heads_linear out", out.dtype), "heads_linear out")
+        if out.shape[0] != n or out_offset < 0 or out_group < N or out_offset + (H - 1) * out_group + N > out.shape[1]:
+            raise KernelError(f"heads_linear: out {tuple(out.shape)} for {n} rows, {H} heads of {N} every {out_group} from "
+                              f"{out_offset}")
+        if n:
+            self._grouped(x, x.stride(0), K, 1, w, out[:, out_offset:], out.stride(0), out_group, None, None, 0, n)
+        return out
+
+    def route_topk(self, z, correction, scale: float, top: int):
+        """A router's choice: (ids [rows, top] int32, weights [rows, top] 32-bit). s = softmax(z) over a row's outputs;
+        the `top` outputs with the largest s + correction are chosen; an output's weight is s * scale."""
+        n, E = z.shape
+        self._f32_rows(z, "router outputs", n, E)
+        if correction is not None:
+            self._f32(correction, "router correction", E)
+        ids = torch.empty(n, top, dtype=torch.int32, device=self.device)
+        weights = torch.empty(n, top, dtype=torch.float32, device=self.device)
+        self._lazy("experts").tis_route_topk(_ptr(z), z.stride(0), _ptr(correction), float(scale), n, E, int(top), _ptr(ids),
+                                             _ptr(weights), self._stream())
+        return ids, weights
+
+    def routed_experts(self, x, ids, weights, w_up, w_down, act: str = "gelu_erf"):
+        """sum_k weights[:, k] * expert(ids[:, k])(x) in 32-bit: expert e < len(w_up) is w_down[e] . act(w_up[e] . x),
+        any id beyond is an identity expert whose result is x itself. x: [rows, width] in the compute type; w_up
+        [experts, hidden, width], w_down [experts, width, hidden]."""
+        _rows_view(self._check(x, "experts x"), "experts x")
+        n, D = x.shape
+        top = ids.shape[1]
+        E = w_up.shape[0] if w_up is not None else 0
+        self._index(ids, "expert ids", n * top)
+        self._f32(weights, "expert weights", n * top)
+        if act != "gelu_erf":
+            raise KernelError(f"routed_experts: activation {act!r} (known: 'gelu_erf')")
+        lib = self._lazy("experts")
+        y = None
+        if E and n:
+            F = w_up.shape[1]
+            if tuple(w_up.shape) != (E, F, D) or tuple(w_down.shape) != (E, D, F):
+                raise KernelError(f"routed_experts: matrices {tuple(w_up.shape)} and {tuple(w_down.shape)} for width {D}")
+            lists = torch.empty(E, n, dtype=torch.int32, device=self.device)
+            counts = torch.empty(E, dtype=torch.int32, device=self.device)
+            lib.tis_expert_lists(_ptr(ids), n * top, E, n, _ptr(lists), _ptr(counts), self._stream())
+            hidden = self.empty(n * top, F)
+            self._grouped(x, x.stride(0), 0, top, w_up, hidden, hidden.stride(0), 0, lists, counts, n, n, act=1)
+            y = torch.empty(n * top, D, dtype=torch.float32, device=self.device)
+            self._grouped(hidden, hidden.stride(0), 0, 1, w_down, y, D, 0, lists, counts, n, n)
+        out = torch.empty(n, D, dtype=torch.float32, device=self.device)
+        lib.tis_experts_combine(self.code, _ptr(y), D, _ptr(x), x.stride(0), _ptr(ids), _ptr(weights), top, E, _ptr(out), D,
+                                n, D, self._stream())
+        return out
+
     # ---- attention with keys and values of different sizes -----------------------------------------------
     def _check_kv_plane(self, plane, n_kv_heads, key_dim, value_dim, page_size):
         self._check(plane, "cache plane")
@@ -1130,18 +1279,24 @@ class HipOps:
                               f"slots x ({key_dim} + {value_dim})")
 
     def attention_prepare(self, proj, q_off, k_off, v_off, positions, write_slots, plane, n_heads, n_kv_heads, key_dim,
-                          value_dim, page_size, q_gain, k_gain, q_factor, freqs, rot_dims, eps, write_cache=True):
+                          value_dim, page_size, q_gain=None, k_gain=None, q_factor=None, freqs=None, rot_dims=0, eps=0.0,
+                          write_cache=True, value_norm=True, q_bias=None, k_bias=None, v_bias=None, temp_coef=0.0,
+                          temp_every=1):
         """From a row's 32-bit projections (queries at column q_off, keys at k_off, values at v_off): queries
-        [rows, heads*key_dim] in the compute type, normed per head (RMS, gain), rotated in interleaved pairs over the
-        first rot_dims channels (angle = position * freqs[pair]) and multiplied by q_factor[head]; keys normed and
-        rotated alike and values divided by their root mean square go into the pages at write_slots."""
+        [rows, heads*key_dim] in the compute type; keys and values go into the pages at write_slots. On the way, each
+        where its argument is given: biases are added; queries and keys are normed per head (RMS, gain of key_dim
+        entries); the first rot_dims channels are rotated in interleaved pairs (angle = position * freqs[pair]);
+        queries are multiplied by q_factor[head] and by 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1);
+        values are divided by their root mean square (value_norm)."""
         n = proj.shape[0]
         need = max(q_off + n_heads * key_dim, k_off + n_kv_heads * key_dim, v_off + n_kv_heads * value_dim)
         self._f32_rows(proj, "attention_prepare projections", n, need)
         self._index(positions, "positions", n)
-        self._f32(q_gain, "query norm gain", key_dim)
-        self._f32(k_gain, "key norm gain", key_dim)
-        self._f32(q_factor, "query factors", n_heads)
+        for t, what, size in ((q_gain, "query norm gain", key_dim), (k_gain, "key norm gain", key_dim),
+                              (q_factor, "query factors", n_heads), (q_bias, "query bias", n_heads * key_dim),
+                              (k_bias, "key bias", n_kv_heads * key_dim), (v_bias, "value bias", n_kv_heads * value_dim)):
+            if t is not None:
+                self._f32(t, what, size)
         if rot_dims:
             self._f32(freqs, "rotary frequencies", rot_dims // 2)
         if write_cache:
@@ -1151,19 +1306,61 @@ class HipOps:
         self._lazy("attention_window").tis_attention_prepare(
             self.code, _ptr(proj), proj.stride(0), q_off, k_off, v_off, _ptr(positions),
             _ptr(write_slots if write_cache else None), _ptr(plane if write_cache else None), _ptr(q), q.stride(0),
-            _ptr(q_gain), _ptr(k_gain), _ptr(q_factor), _ptr(freqs if rot_dims else None), int(rot_dims), float(eps), n,
-            n_heads, n_kv_heads, key_dim, value_dim, page_size, self._stream())
+            _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), _ptr(q_gain), _ptr(k_gain), _ptr(q_factor),
+            _ptr(freqs if rot_dims else None), int(rot_dims), float(eps), 1 if value_norm else 0, float(temp_coef),
+            int(temp_every), n, n_heads, n_kv_heads, key_dim, value_dim, page_size, self._stream())
         return q
 
+    def latent_prepare(self, proj, q_off, c_off, positions, write_slots, plane, n_heads, dim, rot_dim, rank, page_size,
+                       gain, freqs, rot_dims, eps, write_cache=True):
+        """The step before attention over a shared latent. A row's 32-bit projections hold, from column q_off, its
+        query heads as [dim unrotated | rot_dim rotated] each, and from c_off the latent (rank channels) followed by
+        one rotated key part (rot_dim). Returns (q [rows, heads * (rank + rot_dim)] with every head's rotated part in
+        place behind `rank` columns that the caller fills, q_plain [rows, heads * dim]: the unrotated parts), both in
+        the compute type. The latent, RMS-normed with `gain`, and the rotated key part go into the pages at
+        write_slots as keys of rank + rot_dim channels. Rotation: interleaved pairs of the first rot_dims channels
+        of the rotated parts, angle = position * freqs[pair]."""
+        n = proj.shape[0]
+        self._f32_rows(proj, "latent_prepare projections", n, max(q_off + n_heads * (dim + rot_dim), c_off + rank + rot_dim))
+        self._index(positions, "positions", n)
+        self._f32(gain, "latent norm gain", rank)
+        if rot_dims:
+            self._f32(freqs, "rotary frequencies", rot_dims // 2)
+        if write_cache:
+            self._index(write_slots, "write_slots", n)
+            self._check_latent_plane(plane, rank + rot_dim, page_size)
+        q = self.empty(n, n_heads * (rank + rot_dim))
+        q_plain = self.empty(n, n_heads * max(dim, 1))
+        self._lazy("attention_window").tis_latent_prepare(
+            self.code, _ptr(proj), proj.stride(0), q_off, c_off, _ptr(positions), _ptr(write_slots if write_cache else None),
+            _ptr(plane if write_cache else None), _ptr(q), q.stride(0), _ptr(q_plain), q_plain.stride(0), _ptr(gain),
+            _ptr(freqs if rot_dims else None), int(rot_dims), float(eps), n, n_heads, dim, rot_dim, rank, page_size,
+            self._stream())
+        return q, q_plain
+
+    def _check_latent_plane(self, plane, key_dim, page_size):
+        self._check(plane, "cache plane")
+        if not plane.is_contiguous() or plane.shape[0] < 1 or plane.numel() != plane.shape[0] * page_size * key_dim:
+            raise KernelError(f"cache plane {tuple(plane.shape)} does not hold pages of {page_size} slots x {key_dim}")
+
     def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
-                           scale=None):
+                           scale=None, sink=False, gate=None, latent=False):
         """Attention of the rows in `batch` over pages whose keys have key_dim and whose values value_dim channels:
-        [rows, heads*value_dim]."""
+        [rows, heads*value_dim]. sink: the softmax's denominator also counts a key of score 0 that has no value.
+        gate: [rows, heads] 32-bit (a strided view is fine); head h's result is multiplied by sigmoid(gate[:, h]).
+        latent: the pages hold keys only and a key's first value_dim channels are its value (one key/value head)."""
         _rows_view(self._check(q, "q"), "q")
         n = q.shape[0]
-        self._check_kv_plane(plane, n_kv_heads, key_dim, value_dim, page_size)
+        if latent:
+            if n_kv_heads != 1 or value_dim > key_dim:
+                raise KernelError(f"attention over a latent: one key/value head, value {value_dim} <= key {key_dim}")
+            self._check_latent_plane(plane, key_dim, page_size)
+        else:
+            self._check_kv_plane(plane, n_kv_heads, key_dim, value_dim, page_size)
         if q.shape[1] != n_heads * key_dim:
             raise KernelError(f"attention: q width {q.shape[1]} is not heads {n_heads} x key size {key_dim}")
+        if gate is not None:
+            self._f32_rows(gate, "attention gate", n, n_heads)
         tables = batch.block_tables[group]
         self._check(tables, "block tables", torch.int32)
         if tables.dim() != 2 or tables.stride(1) != 1:
@@ -1177,7 +1374,8 @@ class HipOps:
         self._lazy("attention_window").tis_attention_window(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, key_dim, value_dim, page_size,
-            int(window), float(scale if scale is not None else key_dim ** -0.5), self._stream())
+            int(window), float(scale if scale is not None else key_dim ** -0.5), 1 if sink else 0, _ptr(gate),
+            gate.stride(0) if gate is not None else 0, 1 if latent else 0, self._stream())
         return out
 
     # ---- recurrent mixers with a matrix state per head ---------------------------------------------------

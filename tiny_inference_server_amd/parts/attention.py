@@ -172,3 +172,143 @@ class WindowedQkNormAttention:
             self._w_in = to_compute(self.ops, self.input_rows)
         proj = self.ops.linear(x, self._w_in, out_dtype=torch.float32)
         return self.ops.linear(self.core(proj, ctx), self.w_o, residual=residual)
+
+
+def _rotary_frequencies(ops, dims: int, base: float):
+    """base^(-2i/dims) for the pairs i < dims/2, on the device in 32-bit (computed in 64-bit)."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / max(1, dims))).to(torch.float32).to(ops.device)
+
+
+@MIXERS.register("sink_gated_attention")
+class SinkGatedAttention:
+    """Grouped-query attention over all earlier positions with biased projections, no rotation, a query factor that
+    grows with the position, a sink in the softmax and a gate per head.
+
+    q = x.Wq^T + bq, k = x.Wk^T + bk, v = x.Wv^T + bv; the query at position p is multiplied by
+    1 + temp_coef * ln(floor((p + 1) / temp_every) + 1); score = q.k * scale; the weights of a row are
+    exp(s_j) / (1 + sum_j exp(s_j)) (a sink of score 0 without a value); head h's result is multiplied by
+    sigmoid(x.Wg^T)[h]; out = heads . Wo^T. Factors, scores, weights and gates are 32-bit. Keys and values may differ in
+    size.
+
+    params: width, n_heads, n_kv_heads, key_dim, value_dim, scale, temp_coef, temp_every (temp_coef 0: no factor),
+    sink (default true), head_gate (default true). tensors, stored [out, in]: q (heads*key_dim, width), k
+    (kv_heads*key_dim, width), v (kv_heads*value_dim, width), q_bias, k_bias, v_bias, g (heads, width; with head_gate),
+    o (width, heads*value_dim).
+    """
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, H, G, kd, vd = (params[k] for k in ("width", "n_heads", "n_kv_heads", "key_dim", "value_dim"))
+        shapes = {"q": (H * kd, w), "k": (G * kd, w), "v": (G * vd, w), "q_bias": (H * kd,), "k_bias": (G * kd,),
+                  "v_bias": (G * vd,), "o": (w, H * vd)}
+        if params.get("head_gate", True):
+            shapes["g"] = (H, w)
+        return shapes
+
+    @classmethod
+    def cache_need(cls, params):
+        return PagedKvNeed(params["n_kv_heads"], params["key_dim"], 0, value_dim=params["value_dim"])
+
+    def __init__(self, spec, tensors, ops):
+        from .base import to_gain
+        p = spec.params
+        self.ops = ops
+        self.H, self.G, self.kd, self.vd = int(p["n_heads"]), int(p["n_kv_heads"]), int(p["key_dim"]), int(p["value_dim"])
+        if self.H % self.G:
+            raise ValueError(f"{self.H} query heads are not a multiple of {self.G} key/value heads")
+        self.scale = float(p["scale"])
+        self.temp_coef, self.temp_every = float(p.get("temp_coef", 0.0)), int(p.get("temp_every", 1))
+        self.sink, self.head_gate = bool(p.get("sink", True)), bool(p.get("head_gate", True))
+        mats = [tensors.of(spec, k) for k in ("q", "k", "v")] + ([tensors.of(spec, "g")] if self.head_gate else [])
+        self.k_at = mats[0].shape[0]
+        self.v_at = self.k_at + mats[1].shape[0]
+        self.g_at = self.v_at + mats[2].shape[0]
+        self.w_in = to_compute(ops, torch.cat(mats, dim=0))
+        self.q_bias, self.k_bias, self.v_bias = (to_gain(ops, tensors.of(spec, k)) for k in ("q_bias", "k_bias", "v_bias"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+
+    def core(self, x, ctx):
+        ops, b = self.ops, ctx.batch
+        proj = ops.linear(x, self.w_in, out_dtype=torch.float32)
+        q = ops.attention_prepare(proj, 0, self.k_at, self.v_at, b.positions, b.write_slots[ctx.group], ctx.plane, self.H,
+                                  self.G, self.kd, self.vd, ctx.page_size, write_cache=ctx.writes_cache, value_norm=False,
+                                  q_bias=self.q_bias, k_bias=self.k_bias, v_bias=self.v_bias, temp_coef=self.temp_coef,
+                                  temp_every=self.temp_every)
+        gate = proj[:, self.g_at:self.g_at + self.H] if self.head_gate else None
+        return ops.paged_attention_kv(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, self.vd, ctx.page_size, 0,
+                                      self.scale, sink=self.sink, gate=gate)
+
+    def forward32(self, x, ctx):
+        return self.ops.linear(self.core(x, ctx), self.w_o, out_dtype=torch.float32)
+
+    def forward(self, x, ctx, residual=None):
+        return self.ops.linear(self.core(x, ctx), self.w_o, residual=residual)
+
+
+@MIXERS.register("latent_attention")
+class LatentAttention:
+    """Softmax attention whose keys and values are made from one low-rank latent per position.
+
+    q = x.Wq^T, a head being [dim unrotated | rot_dim rotated] channels. x.Wdkv^T gives rank + rot_dim channels: the
+    first rank, RMS-normed with a gain, are the latent c; the others are one rotated key part that all heads share.
+    Head h's unrotated key is Wuk[h] c and its value Wuv[h] c; score = (q_plain . k_plain + q_rot . k_rot) * scale;
+    rotation in interleaved pairs of the first rot_dims channels of the rotated parts by position * base^(-2i/rot_dims);
+    causal softmax; out = heads . Wo^T.
+
+    Only c and the rotated key part are kept, as one key of rank + rot_dim channels per position. The products with
+    Wuk and Wuv are moved to the query's side of the sums: q_plain . (Wuk[h] c) = (Wuk[h]^T q_plain) . c, so a row's
+    query becomes [Wuk[h]^T q_plain | q_rot] against the key [c | k_rot]; and sum_j p_j Wuv[h] c_j = Wuv[h] sum_j p_j c_j,
+    so the attention's values are the latents themselves and Wuv[h] is applied to the result.
+
+    params: width, n_heads, dim, rot_dim, value_dim, rank, rot_dims, rot_base, scale, eps. tensors, stored [out, in]:
+    q (heads*(dim+rot_dim), width), dkv (rank+rot_dim, width), dkv_norm (rank,), uk (heads*dim, rank),
+    uv (heads*value_dim, rank), o (width, heads*value_dim).
+    """
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, H, D, R, V, C = (params[k] for k in ("width", "n_heads", "dim", "rot_dim", "value_dim", "rank"))
+        return {"q": (H * (D + R), w), "dkv": (C + R, w), "dkv_norm": (C,), "uk": (H * D, C), "uv": (H * V, C),
+                "o": (w, H * V)}
+
+    @classmethod
+    def cache_need(cls, params):
+        return PagedKvNeed(1, params["rank"] + params["rot_dim"], 0, value_dim=params["rank"], values_in_keys=True)
+
+    def __init__(self, spec, tensors, ops):
+        from .base import to_gain
+        p = spec.params
+        self.ops = ops
+        self.H, self.D, self.R, self.V, self.C = (int(p[k]) for k in ("n_heads", "dim", "rot_dim", "value_dim", "rank"))
+        self.rot_dims = int(p.get("rot_dims", self.R))
+        if self.rot_dims % 2 or self.rot_dims > self.R:
+            raise ValueError(f"{self.rot_dims} rotated channels of a part of {self.R}: an even number, at most the part")
+        self.scale, self.eps = float(p["scale"]), float(p["eps"])
+        self.freqs = _rotary_frequencies(ops, self.rot_dims, float(p.get("rot_base", 10000.0)))
+        wq, wdkv = tensors.of(spec, "q"), tensors.of(spec, "dkv")
+        self.c_at = wq.shape[0]
+        self.w_in = to_compute(ops, torch.cat((wq, wdkv), dim=0))
+        self.c_gain = to_gain(ops, tensors.of(spec, "dkv_norm"))
+        # [heads, rank, dim]: Wuk[h]^T, which takes a head's unrotated query into the latent's space
+        self.w_uk_t = to_compute(ops, tensors.of(spec, "uk").view(self.H, self.D, self.C).transpose(1, 2))
+        self.w_uv = to_compute(ops, tensors.of(spec, "uv").view(self.H, self.V, self.C))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+
+    def core(self, x, ctx):
+        ops, b = self.ops, ctx.batch
+        H, D, R, V, C = self.H, self.D, self.R, self.V, self.C
+        proj = ops.linear(x, self.w_in, out_dtype=torch.float32)
+        q, q_plain = ops.latent_prepare(proj, 0, self.c_at, b.positions, b.write_slots[ctx.group], ctx.plane, H, D, R, C,
+                                        ctx.page_size, self.c_gain, self.freqs, self.rot_dims, self.eps, ctx.writes_cache)
+        ops.heads_linear(q_plain, self.w_uk_t, q, C + R)
+        mixed = ops.paged_attention_kv(q, ctx.plane, b, ctx.group, H, 1, C + R, C, ctx.page_size, 0, self.scale, latent=True)
+        return ops.heads_linear(mixed, self.w_uv, ops.empty(mixed.shape[0], H * V), V)
+
+    def forward32(self, x, ctx):
+        return self.ops.linear(self.core(x, ctx), self.w_o, out_dtype=torch.float32)
+
+    def forward(self, x, ctx, residual=None):
+        return self.ops.linear(self.core(x, ctx), self.w_o, residual=residual)

@@ -31,6 +31,8 @@ arrangement     part_names (the names of the parts it wires), __init__(layer_spe
 planning        a part may offer plan_key() -> hashable | None and plan_rows(seq_rows, add) -> {name: (array id,
                 host values...)}: host-side work lists for its kernels, made once per step and distinct key while the
                 step's arrays are packed, found again in batch.extras[name]
+token input     forward(x, tokens) -> (y, norm | None): what a block adds to its stream from a table indexed by the rows'
+                tokens; x is the stream in the compute type, y 32-bit, norm = (gain, eps) if y is still to be RMS-normed
 stage input     state_need(params) -> StateNeed | None classmethod
                 forward(batch, previous_output, previous_batch, shared, state) -> rows
 """
@@ -48,6 +50,7 @@ POSITION_ENCODINGS: Registry = Registry("position encoding")
 ARRANGEMENTS: Registry = Registry("block arrangement")
 STAGE_INPUTS: Registry = Registry("stage input")
 GATES: Registry = Registry("residual gate")
+TOKEN_INPUTS: Registry = Registry("per-layer token input")
 
 
 @dataclass
@@ -102,7 +105,7 @@ class Tensors:
 
 
 REGISTRIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "position": POSITION_ENCODINGS,
-              "stage_input": STAGE_INPUTS, "gate": GATES}
+              "stage_input": STAGE_INPUTS, "gate": GATES, "token_input": TOKEN_INPUTS}
 
 
 def part_class(spec):

@@ -36,3 +36,54 @@ class SwiGlu:
             x, norm = norm(x), None
         hidden = ops.linear_swiglu(x, self.w_gate_up, rms=norm.as_rms() if norm is not None else None)
         return ops.linear(hidden, self.w_down, residual=residual, reuse_residual=residual_is_spent)
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts:
+    """A mixture of small feed-forwards of which every row uses `top`.
+
+    z = x.Wr^T (32-bit), s = softmax(z) over all router outputs; the `top` outputs with the largest s + correction are
+    chosen; a chosen output's weight is s * scale (without the correction, not renormalised). Output e < n_experts is
+    the expert Wdown[e] . act(Wup[e] . x) (no biases, act the erf-form gelu); the last n_identity outputs are identity
+    experts without tensors whose result is x itself. y = the weighted sum of the chosen outputs, in 32-bit.
+
+    params: width, hidden, n_experts, n_identity, top, scale. tensors, stored [out, in]: router
+    (n_experts + n_identity, width), correction (n_experts + n_identity,), up<e> (hidden, width), down<e> (width, hidden).
+    """
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, f, E, I = params["width"], params["hidden"], params["n_experts"], params.get("n_identity", 0)
+        shapes = {"router": (E + I, w), "correction": (E + I,)}
+        for e in range(E):
+            shapes[f"up{e}"] = (f, w)
+            shapes[f"down{e}"] = (w, f)
+        return shapes
+
+    def __init__(self, spec, tensors, ops):
+        from .base import to_gain
+        p = spec.params
+        self.ops = ops
+        self.E, self.I, self.top = int(p["n_experts"]), int(p.get("n_identity", 0)), int(p["top"])
+        if not 1 <= self.top <= self.E + self.I:
+            raise ValueError(f"{self.top} of {self.E} + {self.I} experts")
+        self.scale = float(p.get("scale", 1.0))
+        self.w_router = to_compute(ops, tensors.of(spec, "router"))
+        self.correction = to_gain(ops, tensors.of(spec, "correction"))
+        self.w_up = self.w_down = None
+        if self.E:
+            self.w_up = to_compute(ops, torch.stack([tensors.of(spec, f"up{e}") for e in range(self.E)]))
+            self.w_down = to_compute(ops, torch.stack([tensors.of(spec, f"down{e}") for e in range(self.E)]))
+
+    def forward32(self, x):
+        ops = self.ops
+        z = ops.linear(x, self.w_router, out_dtype=torch.float32)
+        ids, weights = ops.route_topk(z, self.correction, self.scale, self.top)
+        return ops.routed_experts(x, ids, weights, self.w_up, self.w_down, "gelu_erf")
+
+    def forward(self, x, residual=None):
+        y = self.forward32(x)
+        if residual is not None:
+            y = y + residual.to(torch.float32)
+        return y.to(self.ops.dtype)

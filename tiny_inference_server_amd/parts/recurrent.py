@@ -119,3 +119,50 @@ class MatrixMemory(_MatrixStateMixer):
         o = ops.state_scan("gated_max", proj, at["q"], at["k"], at["v"], D ** -0.5, ctx.state, ctx.batch, H, D, V,
                            i_off=at["i"], f_off=at["f"], bias_i=self.i_bias, bias_f=self.f_bias, cap=self.cap)
         return ops.head_norm_gate(o, proj[:, at["g"]:at["g"] + H * V], self.norm_gain, H, V, self.eps, "sigmoid")
+
+
+@MIXERS.register("lightning_attention")
+class LightningAttention(_MatrixStateMixer):
+    """Linear attention with one fixed decay per head: q = silu(x.Wq^T), k = silu(x.Wk^T), v = silu(x.Wv^T); per head
+    S_t = decay[h] S_(t-1) + k_t v_t^T, o_t = S_t^T q_t, with no other scale. The heads side by side are RMS-normed
+    together with a gain, multiplied by sigmoid(x.Wg^T) and projected by Wo. State and sums are 32-bit; the state
+    starts at zero.
+
+    params: width, n_heads, dim, vdim, decay (one number per head), eps. tensors, stored [out, in]: q, k
+    (heads*dim, width), v, g (heads*vdim, width), o (width, heads*vdim), norm (heads*vdim,).
+    """
+
+    @classmethod
+    def tensor_shapes(cls, params):
+        w, H, D, V = (params[k] for k in ("width", "n_heads", "dim", "vdim"))
+        return {"q": (H * D, w), "k": (H * D, w), "v": (H * V, w), "g": (H * V, w), "o": (w, H * V), "norm": (H * V,)}
+
+    @classmethod
+    def cache_need(cls, params):
+        return StateNeed((state_floats("decay", params["n_heads"], params["dim"], params["vdim"]),), "float32")
+
+    def __init__(self, spec, tensors, ops):
+        p = spec.params
+        self.ops = ops
+        self.H, self.D, self.V = int(p["n_heads"]), int(p["dim"]), int(p["vdim"])
+        self.eps = float(p["eps"])
+        decay = [float(a) for a in p["decay"]]
+        if len(decay) != self.H:
+            raise ValueError(f"{len(decay)} decays for {self.H} heads")
+        # the scan takes a decay per key channel and row: one line that every row reads
+        self.decay = torch.tensor(decay, dtype=torch.float64).repeat_interleave(self.D).to(torch.float32).to(ops.device).view(1, -1)
+        self.at = self._stack(spec, tensors, ("q", "k", "v", "g"))
+        self.norm_gain = to_gain(ops, tensors.of(spec, "norm"))
+        self.w_o = to_compute(ops, tensors.of(spec, "o"))
+
+    def core(self, proj, ctx):
+        ops, at, H, D, V = self.ops, self.at, self.H, self.D, self.V
+        ops.activate32(proj[:, :at["g"]], "silu")           # q, k and v lie first, side by side
+        o = ops.state_scan("decay", proj, at["q"], at["k"], at["v"], 1.0, ctx.state, ctx.batch, H, D, V,
+                           decay=self.decay.expand(proj.shape[0], H * D))
+        return ops.head_norm_gate(o, proj[:, at["g"]:at["g"] + H * V], self.norm_gain, 1, H * V, self.eps, "sigmoid")
+
+    def forward32(self, x, ctx):
+        if self._w_in is None:
+            self._w_in = to_compute(self.ops, self.input_rows)
+        return self.forward_projected(self.ops.linear(x, self._w_in, out_dtype=torch.float32), ctx)

@@ -21,7 +21,7 @@ from typing import Any, Mapping, Optional, Tuple
 @dataclass(frozen=True)
 class PartSpec:
     role: str                     # which registry `kind` is looked up in: "norm", "position", "mixer",
-                                  # "feed_forward" or "stage_input"
+                                  # "feed_forward", "gate", "token_input" or "stage_input"
     kind: str
     params: Mapping[str, Any] = field(default_factory=dict)    # sizes, constants, nested PartSpecs
     tensors: Mapping[str, str] = field(default_factory=dict)   # local key -> tensor name in the file
@@ -84,11 +84,13 @@ class ModelSpec:
 @dataclass(frozen=True)
 class PagedKvNeed:
     """Keys and values of every position (window 0) or of the last `window` positions. value_dim: channels of a
-    value where they differ from a key's head_dim (0: the same)."""
+    value where they differ from a key's head_dim (0: the same). values_in_keys: nothing is kept beside the keys (a
+    shared latent whose first channels are the values); value_dim then only says how many."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
     value_dim: int = 0
+    values_in_keys: bool = False
 
 
 @dataclass(frozen=True)
