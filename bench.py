@@ -18,8 +18,8 @@ with temperature, top-k, top-p and repetition penalty, finishing, pages given ba
     python bench.py --workload mixed --size 2.1B     64 requests decoding at contexts of 512..8192 while 2,048-token
                                                      portions of further prompts run in the same steps
 
-    python bench.py --workload designs               the Fikevik design beside the grouped-query decoder at equal sizes:
-                                                     prefill and decode throughput of both at a few layer sizes
+    python bench.py --workload designs               the Fikevik and Fipuzen designs beside the grouped-query decoder at equal
+                                                     sizes: prefill and decode throughput of each at a few layer sizes
 
 Each prints one line of the same form; `value` is generated tokens a second over the whole run (serve) or over the
 steps that hold 64 decoding requests and a portion (mixed), `roofline` the sum of the steps' floors (the larger of
@@ -304,9 +304,28 @@ def fikevik_config(width, heads, kv_heads, ff, layers, vocab, window=1024):
                              "layers": [par if i % 2 == 0 else gla for i in range(layers)]})
 
 
+def fipuzen_config(width, heads, kv_heads, ff, layers, vocab, experts=8, top=2):
+    """Attention with a sink, lightning attention and attention over a latent in turn; every layer with a mixture of
+    `experts` experts of which a row takes `top`, each expert ff / top wide, so that a row's feed-forward does the work
+    of a dense one of width ff; a token input of 64 numbers a layer."""
+    from tiny_inference_server_amd.config import config_from_dict
+    mlp = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": experts, "identity": 1, "top": top, "scale": 1.0}}
+    kinds = [{"type": "attention", "mlp": mlp,
+              "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                        "q_temp": {"coef": 0.1, "every": 1024}}},
+             {"type": "lightning", "mlp": mlp,
+              "mixer": {"heads": heads // 2, "dim": 128, "vdim": 256, "decay": [1.0 - 2.0 ** -(5 + i % 6) for i in range(heads // 2)]}},
+             {"type": "latent_attention", "mlp": mlp,
+              "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+                        "rot": {"dims": 64, "base": 1000000.0}}}]
+    return config_from_dict({"architecture": "Fipuzen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+                             "token_side": {"dim": 64}, "layers": [kinds[i % 3] for i in range(layers)]})
+
+
 def design_comparison(a, say):
-    """Prefill (a.prefill_tokens tokens, one prompt) and decode (batch a.batch, context a.context) of the Fikevik design
-    and of the grouped-query decoder without prediction heads at the sizes of DESIGN_SIZES, random weights."""
+    """Prefill (a.prefill_tokens tokens, one prompt) and decode (batch a.batch, context a.context) of the Fikevik and
+    Fipuzen designs and of the grouped-query decoder without prediction heads at the sizes of DESIGN_SIZES, random
+    weights."""
     import torch
 
     from tiny_inference_server_amd.config import GqaMtpConfig
@@ -322,6 +341,7 @@ def design_comparison(a, say):
     for name, width, heads, kv_heads, ff, layers in sizes:
         designs = {
             "fikevik": fikevik_config(width, heads, kv_heads, ff, layers, vocab),
+            "fipuzen": fipuzen_config(width, heads, kv_heads, ff, layers, vocab),
             "gqa": GqaMtpConfig(d_model=width, vocab_size=vocab, max_context=max(8192, a.context), rope_base=500000.0,
                                 n_heads=heads, n_layers=layers, ffn_hidden=ff, group_size=heads // kv_heads, mtp_heads=0,
                                 rms_eps=1e-5, tie_embeddings=False),
@@ -380,7 +400,7 @@ def design_comparison(a, say):
             "warmup": a.warmup, "ms_per_step": points[first].get("decode_ms"), "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": dkey,
             "data": "synthetic: random weights N(0,0.02), uniform random token ids",
-            "config": {"model": "Fikevik beside GqaMtpTransformer", "sizes": [list(s) for s in DESIGN_SIZES],
+            "config": {"model": "Fikevik and Fipuzen beside GqaMtpTransformer", "sizes": [list(s) for s in DESIGN_SIZES],
                        "global_batch": a.batch, "seq_len": a.context, "prefill_tokens": a.prefill_tokens,
                        "parallelism": "single-gpu"},
             "points": points}
@@ -408,7 +428,7 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", choices=["decode", "serve", "mixed", "designs"], default="decode")
     ap.add_argument("--requests", type=int, default=64, help="serve, mixed: requests (decoding at once)")
-    ap.add_argument("--designs", default="", help="designs: which of fikevik,gqa to run (default: both)")
+    ap.add_argument("--designs", default="", help="designs: which of fikevik,fipuzen,gqa to run (default: all)")
     ap.add_argument("--design-sizes", default="", help="designs: which sizes to run, e.g. w2048 (default: all)")
     ap.add_argument("--phase", choices=["both", "prefill", "decode"], default="both", help="designs: what to measure")
     ap.add_argument("--new-tokens", type=int, default=256, help="serve: tokens generated per request")

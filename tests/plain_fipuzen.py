@@ -128,13 +128,21 @@ def latent_attention(h, t, pre, m, eps):
     return out.reshape(T, H * V) @ w64(t, pre + "o").T
 
 
-def routed_experts(h, t, pre, mlp):
-    """Mixture of experts with identity experts at the end of the router's outputs."""
+def routed_experts(h, t, pre, mlp, margins=None):
+    """Mixture of experts with identity experts at the end of the router's outputs. margins (a list) receives, per
+    row, how clear the closest choice was: the gap between the last chosen and the first unchosen score over the larger
+    of the two softmax values (about the change of a router output that would turn the choice)."""
     r = mlp["router"]
     E, I, top = r["experts"], r.get("identity", 0), r["top"]
     z = h @ w64(t, pre + "router").T                                 # [T, E + I]
     s = torch.softmax(z, dim=-1)
-    chosen = torch.topk(s + w64(t, pre + "correction"), top, dim=-1).indices
+    choice = s + w64(t, pre + "correction")
+    chosen = torch.topk(choice, top, dim=-1).indices
+    if margins is not None and top < E + I:
+        order = torch.sort(choice, dim=-1, descending=True)
+        gap = order.values[:, top - 1] - order.values[:, top]
+        big = torch.maximum(torch.gather(s, 1, order.indices[:, top - 1:top]), torch.gather(s, 1, order.indices[:, top:top + 1]))
+        margins.extend((gap / big[:, 0]).tolist())
     out = torch.zeros_like(h)
     for i in range(h.shape[0]):
         for e in chosen[i].tolist():
@@ -153,7 +161,7 @@ def token_side(x, tokens, t, pre, layer, dim, eps):
     return rms_norm(y, w64(t, pre + "norm"), eps)
 
 
-def forward(cfg, t, tokens, layer_outputs=None):
+def forward(cfg, t, tokens, layer_outputs=None, margins=None):
     """Logits [T, vocab] in float64 for one sequence. cfg: the raw dictionary of config.json; t: tensors by name."""
     eps = cfg["norm"]["eps"]
     tokens = torch.as_tensor(tokens, dtype=torch.int64)
@@ -172,10 +180,17 @@ def forward(cfg, t, tokens, layer_outputs=None):
             raise ValueError(entry["type"])
         if entry.get("mlp") is not None:
             h = layer_norm(x, w64(t, pre + "norm2"), w64(t, pre + "norm2.b"), eps)
-            x = x + routed_experts(h, t, pre + "mlp.", entry["mlp"])
+            x = x + routed_experts(h, t, pre + "mlp.", entry["mlp"], margins)
         if side:
             x = x + token_side(x, tokens, t, pre + "side.", i, side["dim"], eps)
         if layer_outputs is not None:
             layer_outputs.append(x.clone())
     x = layer_norm(x, w64(t, "final.norm"), w64(t, "final.norm.b"), eps)
     return x @ w64(t, "head").T
+
+
+def greedy_generate(cfg, t, prompt, n_new):
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(torch.argmax(forward(cfg, t, ids)[-1])))
+    return ids[len(prompt):]

@@ -120,7 +120,8 @@ class TorchOps:
             plane[:, 1] = vt.reshape(plane.shape[0], n_kv_heads, page_size, head_dim)
 
     # ---- attention over the paged cache -----------------------------------------------------------------
-    def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None, slopes=None):
+    def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None, slopes=None,
+                        sink=False, gate=None):
         n = q.shape[0]
         page_size = plane.shape[3]
         scale = scale if scale is not None else head_dim ** -0.5
@@ -142,8 +143,17 @@ class TorchOps:
                 s = (k[:, h // g] @ qr[h]) * scale
                 if slopes is not None:
                     s = s + float(slopes[h]) * (js - p).float()
-                out[r, h * head_dim:(h + 1) * head_dim] = torch.softmax(s, dim=0) @ v[:, h // g]
+                w = torch.softmax(torch.cat((s, s.new_zeros(1))), dim=0)[:-1] if sink else torch.softmax(s, dim=0)
+                o = w @ v[:, h // g]
+                if gate is not None:
+                    o = o * torch.sigmoid(gate[r, h].float())
+                out[r, h * head_dim:(h + 1) * head_dim] = o
         return out.to(q.dtype)
+
+    def head_gate(self, x, gate, n_heads, vdim):
+        y = x.float().view(x.shape[0], n_heads, vdim) * torch.sigmoid(gate.float())[:, :, None]
+        x.copy_(y.view(x.shape[0], n_heads * vdim).to(x.dtype))
+        return x
 
     # ---- a residual stream in 32-bit, norm after the sum ---------------------------------------------------
     def embed_scaled(self, table, tokens, scale):

@@ -18,6 +18,14 @@ int tis_attention_mfma(const void* q, long q_ld, const void* plane, const int* b
                        int n_heads, int n_kv_heads, int head_dim, int page_size, int window, float scale, int n_splits,
                        int min_steps, int tile_splits, int tile_max_steps, int* row_splits, hipStream_t stream);
 
+// tis_attention_mfma with a sink in every row's softmax where sink != 0 (one more key of score 0 without a value).
+int tis_attention_mfma_sink(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
+                            const int* row_seq, const int* positions, const int* items, int n_items, int nb,
+                            const int* tiles, int n_tiles, void* out, long out_ld, float* part_o, float* part_ml, int rows,
+                            int n_heads, int n_kv_heads, int head_dim, int page_size, int window, float scale, int n_splits,
+                            int min_steps, int tile_splits, int tile_max_steps, int* row_splits, int sink,
+                            hipStream_t stream);
+
 // A second stream (default priority, as `stream` must have) on which a call that holds both tiles and items runs its
 // tile kernel, beside the items' kernel on `stream`; the two meet again before the merge, and everything after the
 // call on `stream` waits for both. Per device; null (the start) keeps everything on `stream`. The stream must outlive

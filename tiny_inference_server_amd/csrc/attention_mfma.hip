@@ -77,7 +77,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ items,
     bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
     int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int min_steps,
-    int split_stride, int* __restrict__ row_splits) {
+    int split_stride, int* __restrict__ row_splits, int sink) {
   const int page_size = PS16 ? 16 : page_size_arg;
   const int item = blockIdx.x, kvh = blockIdx.y;
   int split = blockIdx.z;
@@ -347,7 +347,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NB <= 2 ? 2 
     const float lt = column_sum(l[nb]);
     if (!col_ok[nb]) continue;
     if (item_splits == 1) {
-      const float inv = 1.f / lt;
+      // a sink: one more key of score 0 without a value, which only the denominator sees
+      const float inv = 1.f / (sink ? lt + __builtin_amdgcn_exp2f(-m[nb]) : lt);
       bf16* dst = out + (long)col_row[nb] * out_ld + (long)col_head[nb] * HD + g * 4;
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
@@ -433,7 +434,7 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(HD <= 1
     int bt_ld, const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ tiles,
     bf16* __restrict__ out, long out_ld, float* __restrict__ part_o, float2* __restrict__ part_ml, int group_size,
     int n_kv_heads, int n_heads, int page_size_arg, int window, float scale_log2, int n_splits, int max_steps,
-    int split_stride, int* __restrict__ row_splits) {
+    int split_stride, int* __restrict__ row_splits, int sink) {
   __shared__ __attribute__((aligned(16))) bf16 k_lds[TBUF][TCH * 8];
   __shared__ __attribute__((aligned(16))) bf16 v_lds[TBUF][TCH * 8];
   const int page_size = PS16 ? 16 : page_size_arg;
@@ -707,7 +708,7 @@ __global__ __launch_bounds__(TW * 64) __attribute__((amdgpu_waves_per_eu(HD <= 1
   const float lt = pair_sum(l);
   if (!col_ok) return;
   if (item_splits == 1) {
-    const float inv = 1.f / lt;
+    const float inv = 1.f / (sink ? lt + __builtin_amdgcn_exp2f(-m) : lt);
     bf16* dst = out + (long)col_row * out_ld + (long)col_head * HD + h * 4;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -742,7 +743,8 @@ static constexpr int MD = (HD + 63) / 64;  // outputs per lane
 __global__ __launch_bounds__(MG * 64) void attention_merge_kernel(const float* __restrict__ part_o,
                                                                   const float2* __restrict__ part_ml,
                                                                   bf16* __restrict__ out, long out_ld, int n_heads,
-                                                                  int max_splits, const int* __restrict__ row_splits) {
+                                                                  int max_splits, const int* __restrict__ row_splits,
+                                                                  int sink) {
   __shared__ float so[MG][MD][64];
   const long row = blockIdx.x;
   const int head = blockIdx.y;
@@ -792,6 +794,7 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_kernel(const float* _
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+  if (sink) L += exp2f(-M);      // the sink's share of the denominator, once for all splits
 #pragma unroll
   for (int j = 0; j < MD; ++j) so[grp][j][lane] = acc[j];
   __syncthreads();
@@ -815,7 +818,7 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_rows_kernel(const flo
                                                                        const float2* __restrict__ part_ml,
                                                                        bf16* __restrict__ out, long out_ld,
                                                                        int n_heads, int max_splits,
-                                                                       const int* __restrict__ row_splits) {
+                                                                       const int* __restrict__ row_splits, int sink) {
   const long row = blockIdx.x;
   const int n_splits = row_splits ? row_splits[row] : max_splits;
   if (n_splits <= 1) return;
@@ -852,6 +855,7 @@ __global__ __launch_bounds__(MG * 64) void attention_merge_rows_kernel(const flo
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+  if (sink) L += exp2f(-M);
 #pragma unroll
   for (int j = 0; j < MD; ++j) {
     const int d = j * 64 + lane;
@@ -916,7 +920,7 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
                             const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
                             float* part_ml, int rows, int n_heads, int n_kv_heads, int head_dim, int page_size,
                             int window, float scale, int n_splits, int min_steps, int tile_splits,
-                            int tile_max_steps, int* row_splits, hipStream_t stream) {
+                            int tile_max_steps, int* row_splits, hipStream_t stream, int sink = 0) {
   if ((n_items == 0 && n_tiles == 0) || rows == 0) return 0;
   if (n_items < 0 || n_tiles < 0 || (n_tiles > 0 && !tiles)) return tis_fail("attention_mfma: bad item counts %d, %d", n_items, n_tiles);
   if (head_dim != HD) return tis_fail("attention_mfma: built for head size %d, called with %d", HD, head_dim);
@@ -976,7 +980,7 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   attention_mfma_kernel<NBV, PSV><<<grid, 64, 0, stream>>>(                                                      \
       (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)items,     \
       (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
-      n_splits, min_steps, stride, row_splits)
+      n_splits, min_steps, stride, row_splits, sink)
     if (page_size == 16) {
       if (nb == 1) LAUNCH(1, true);
       else if (nb == 2) LAUNCH(2, true);
@@ -995,7 +999,7 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
   attention_tile_kernel<PSV><<<grid, TW * 64, 0, tile_stream>>>(                                                      \
       (const bf16*)q, q_ld, (const bf16*)plane, block_tables, bt_ld, row_seq, positions, (const int2*)tiles,     \
       (bf16*)out, out_ld, part_o, (float2*)part_ml, group, n_kv_heads, n_heads, page_size, window, scale_log2,   \
-      tile_splits, tile_max_steps, stride, row_splits)
+      tile_splits, tile_max_steps, stride, row_splits, sink)
     if (page_size == 16) LAUNCH(true);
     else LAUNCH(false);
 #undef LAUNCH
@@ -1009,11 +1013,11 @@ static int attention_launch(const void* q, long q_ld, const void* plane, const i
     if ((long)rows * n_heads > 8192) {
       dim3 mgrid(rows, (n_heads + MG - 1) / MG);
       attention_merge_rows_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,
-                                                                 n_heads, stride, row_splits);
+                                                                 n_heads, stride, row_splits, sink);
     } else {
       dim3 mgrid(rows, n_heads);
       attention_merge_kernel<<<mgrid, MG * 64, 0, stream>>>(part_o, (const float2*)part_ml, (bf16*)out, out_ld,
-                                                            n_heads, stride, row_splits);
+                                                            n_heads, stride, row_splits, sink);
     }
     rc = tis_launch_status("attention_merge");
   }
@@ -1029,6 +1033,19 @@ TIS_EXPORT int tis_attention_mfma(const void* q, long q_ld, const void* plane, c
   return attention_launch(q, q_ld, plane, block_tables, bt_ld, row_seq, positions, items, n_items, nb, tiles, n_tiles,
                           out, out_ld, part_o, part_ml, rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
                           n_splits, min_steps, tile_splits, tile_max_steps, row_splits, stream);
+}
+
+// The same with a sink in every row's softmax (sink != 0): the denominator also counts one key of score 0 that has no
+// value, so a row's weights add up to less than one.
+TIS_EXPORT int tis_attention_mfma_sink(const void* q, long q_ld, const void* plane, const int* block_tables, int bt_ld,
+                                       const int* row_seq, const int* positions, const int* items, int n_items, int nb,
+                                       const int* tiles, int n_tiles, void* out, long out_ld, float* part_o,
+                                       float* part_ml, int rows, int n_heads, int n_kv_heads, int head_dim, int page_size,
+                                       int window, float scale, int n_splits, int min_steps, int tile_splits,
+                                       int tile_max_steps, int* row_splits, int sink, hipStream_t stream) {
+  return attention_launch(q, q_ld, plane, block_tables, bt_ld, row_seq, positions, items, n_items, nb, tiles, n_tiles,
+                          out, out_ld, part_o, part_ml, rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                          n_splits, min_steps, tile_splits, tile_max_steps, row_splits, stream, sink);
 }
 
 // ---- the same without a workspace argument: partial results in memory that this library owns for good ----

@@ -232,6 +232,18 @@ __global__ __launch_bounds__(S32_THREADS) void activate32_kernel(float* __restri
   *p = act == 0 ? gelu_tanh_f(v) : act == 1 ? v * sigmoid_f(v) : sigmoid_f(v);
 }
 
+// x[r][h * V + j] *= sigmoid(gate[r][h]), in place
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void head_gate_kernel(T* __restrict__ x, long ldx, const float* __restrict__ gate,
+                                                                 long ldg, int rows, int H, int V) {
+  const long i = (long)blockIdx.x * S32_THREADS + threadIdx.x;
+  const long W = (long)H * V;
+  if (i >= rows * W) return;
+  const long r = i / W;
+  const int c = (int)(i % W);
+  x[r * ldx + c] = from_f<T>(to_f(x[r * ldx + c]) * sigmoid_f(gate[r * ldg + c / V]));
+}
+
 #define S32_DISPATCH(call_f32, call_bf16)                 \
   if (dtype == TIS_F32) { call_f32; }                     \
   else if (dtype == TIS_BF16) { call_bf16; }              \
@@ -333,4 +345,14 @@ TIS_EXPORT int tis_activate32(float* z, long ldz, int act, int rows, int W, hipS
   const long blocks = ((long)rows * W + S32_THREADS - 1) / S32_THREADS;
   activate32_kernel<<<blocks, S32_THREADS, 0, stream>>>(z, ldz, act, rows, W);
   return tis_launch_status("activate32");
+}
+
+TIS_EXPORT int tis_head_gate(int dtype, void* x, long ldx, const float* gate, long ldg, int rows, int H, int V,
+                             hipStream_t stream) {
+  if (rows == 0) return 0;
+  if (rows < 0 || H < 1 || V < 1) return tis_fail("head_gate: bad size rows=%d heads=%d vdim=%d", rows, H, V);
+  const long blocks = ((long)rows * H * V + S32_THREADS - 1) / S32_THREADS;
+  S32_DISPATCH((head_gate_kernel<float><<<blocks, S32_THREADS, 0, stream>>>((float*)x, ldx, gate, ldg, rows, H, V)),
+               (head_gate_kernel<bf16><<<blocks, S32_THREADS, 0, stream>>>((bf16*)x, ldx, gate, ldg, rows, H, V)))
+  return tis_launch_status("head_gate");
 }

@@ -99,6 +99,8 @@ _SIGNATURES["attention_mfma"] = ("tis_attention_mfma", {
     "tis_attention_mfma_side_stream": [_P],
     "tis_attention_mfma": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F,
                            _I, _I, _I, _I, _P, _P],
+    "tis_attention_mfma_sink": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _I, _P, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F,
+                                _I, _I, _I, _I, _P, _I, _P],
 })
 
 _SIGNATURES["stream32"] = ("tis_stream32", {
@@ -111,6 +113,7 @@ _SIGNATURES["stream32"] = ("tis_stream32", {
     "tis_residual_norm": [_I, _P, _P, _L, _P, _F, _P, _P, _L, _I, _P, _P, _F, _P, _L, _I, _I, _P],
     "tis_gate_table": [_I, _P, _L, _P, _L, _P, _I, _P, _L, _I, _I, _P],
     "tis_activate32": [_P, _L, _I, _I, _I, _P],
+    "tis_head_gate": [_I, _P, _L, _P, _L, _I, _I, _I, _P],
 })
 _SIGNATURES["attention_window"] = ("tis_attention_window", {
     "tis_attention_prepare": [_I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _F, _I,
@@ -917,13 +920,18 @@ class HipOps:
                               f"{head_dim}] contiguous")
 
     def paged_attention(self, q, plane, batch, group, n_heads, n_kv_heads, head_dim, window=0, scale=None,
-                        slopes=None):
+                        slopes=None, sink=False, gate=None):
         """Attention of the rows in `batch` over the cache plane; `q` is [rows, heads*head_dim] (a strided view is fine).
 
         `batch` brings positions, row_seq and the group's block tables; `group` names the page group. `slopes`
         ([heads] 32-bit, or None): a bias slope[h] * (key position - row position) on the scores; such calls go to
-        the general kernel.
+        the general kernel. sink: the softmax's denominator also counts a key of score 0 that has no value. gate
+        ([rows, heads] 32-bit, a strided view is fine): head h's result is multiplied by sigmoid(gate[:, h]). Calls with
+        a sink or a gate that the matrix-core kernels do not take go to the kernel for keys and values of any sizes.
         """
+        group_name = group
+        if (sink or gate is not None) and slopes is not None:
+            raise KernelError("attention: score slopes go with neither a sink nor a gate")
         _rows_view(self._check(q, "q"), "q")
         n = q.shape[0]
         page_size = plane.shape[3]
@@ -1021,12 +1029,17 @@ class HipOps:
                     row_splits = self._workspace[lp.row_splits_offset:]
             if lines.dtype != torch.int32 or not lines.is_contiguous():
                 raise KernelError("attention: the work list must be contiguous 32-bit integers")
-            lib.tis_attention_mfma(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),
-                                   _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(tiles),
-                                   n_tiles, _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads,
-                                   n_kv_heads, head_dim, page_size, int(window), float(scale), n_splits, min_steps,
-                                   tile_splits, tile_max_steps, _ptr(row_splits), self._stream())
+            lib.tis_attention_mfma_sink(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0),
+                                        _ptr(batch.row_seq), _ptr(batch.positions), _ptr(items), n_items, nb, _ptr(tiles),
+                                        n_tiles, _ptr(out), out.stride(0), _ptr(part_o), _ptr(part_ml), n, n_heads,
+                                        n_kv_heads, head_dim, page_size, int(window), float(scale), n_splits, min_steps,
+                                        tile_splits, tile_max_steps, _ptr(row_splits), 1 if sink else 0, self._stream())
+            if gate is not None:
+                self.head_gate(out, gate, n_heads, head_dim)
             return out
+        if sink or gate is not None:
+            return self.paged_attention_kv(q, plane, batch, group_name, n_heads, n_kv_heads, head_dim, head_dim, page_size,
+                                           window, scale, sink=sink, gate=gate)
         self.attn_generic.tis_attention_generic(
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, head_dim, page_size, int(window),
@@ -1191,6 +1204,18 @@ class HipOps:
         self._lazy("stream32").tis_gate_table(self.code, _ptr(z), z.stride(0), _ptr(table), table.stride(0), _ptr(tokens),
                                               self._ACTS[act], _ptr(out), out.stride(0), n, W, self._stream())
         return out
+
+    def head_gate(self, x, gate, n_heads: int, vdim: int):
+        """x[:, h * vdim + (0..vdim)] *= sigmoid(gate[:, h]), in place. x: [rows, heads * vdim] in the compute type;
+        gate: [rows, heads] 32-bit (a strided view is fine)."""
+        _rows_view(self._check(x, "head_gate x"), "head_gate x")
+        n = x.shape[0]
+        if x.shape[1] != n_heads * vdim:
+            raise KernelError(f"head_gate: x {tuple(x.shape)} for {n_heads} heads of {vdim}")
+        self._f32_rows(gate, "head_gate gate", n, n_heads)
+        self._lazy("stream32").tis_head_gate(self.code, _ptr(x), x.stride(0), _ptr(gate), gate.stride(0), n, n_heads, vdim,
+                                             self._stream())
+        return x
 
     def activate32(self, z, act: str):
         """act on 32-bit rows, in place (z may be a strided view of some columns)."""

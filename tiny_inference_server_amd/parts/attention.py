@@ -228,6 +228,20 @@ class SinkGatedAttention:
         self.w_in = to_compute(ops, torch.cat(mats, dim=0))
         self.q_bias, self.k_bias, self.v_bias = (to_gain(ops, tensors.of(spec, k)) for k in ("q_bias", "k_bias", "v_bias"))
         self.w_o = to_compute(ops, tensors.of(spec, "o"))
+        self.same = self.kd == self.vd        # then the pages have the layout every attention kernel reads
+
+    # the matrix-core kernels' work lists, where keys and values are of one size (see GqaAttention)
+    def plan_key(self):
+        if not self.same or not hasattr(self.ops, "plan_attention"):
+            return None
+        return ("attention", self.H, self.G, self.kd, 0)
+
+    def plan_mode(self, seq_rows):
+        mode = getattr(self.ops, "plan_attention_mode", None)
+        return mode(seq_rows, 0) if mode is not None and self.same else None
+
+    def plan_rows(self, seq_rows, add, mode=None):
+        return self.ops.plan_attention(self.H, self.G, self.kd, seq_rows, add, mode, 0)
 
     def core(self, x, ctx):
         ops, b = self.ops, ctx.batch
@@ -237,6 +251,9 @@ class SinkGatedAttention:
                                   q_bias=self.q_bias, k_bias=self.k_bias, v_bias=self.v_bias, temp_coef=self.temp_coef,
                                   temp_every=self.temp_every)
         gate = proj[:, self.g_at:self.g_at + self.H] if self.head_gate else None
+        if self.same:
+            return ops.paged_attention(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, 0, self.scale, sink=self.sink,
+                                       gate=gate)
         return ops.paged_attention_kv(q, ctx.plane, b, ctx.group, self.H, self.G, self.kd, self.vd, ctx.page_size, 0,
                                       self.scale, sink=self.sink, gate=gate)
 
