@@ -125,20 +125,23 @@ def test_attention_with_bias_sink_query_factor_and_head_gate(dtype, Hq, G, kd, v
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("Hq,D,R,V,C,dims", [(3, 16, 8, 12, 24, 8), (2, 5, 6, 7, 300, 4), (8, 64, 32, 64, 128, 32), (1, 12, 0, 9, 40, 0)])
+@pytest.mark.parametrize("Hq,D,R,V,C,dims", [(3, 16, 8, 12, 24, 8), (2, 5, 6, 7, 300, 4), (8, 64, 32, 64, 128, 32), (1, 12, 0, 9, 40, 0),
+                                             (20, 24, 16, 8, 48, 16), (16, 128, 64, 128, 512, 64)])
 def test_attention_over_a_latent(dtype, Hq, D, R, V, C, dims):
     """The step before (norm of the latent, rotation, the pages), the product per head into the latent's space, the
-    attention whose values are part of its keys, and the product per head back out."""
+    attention whose values are part of its keys, and the product per head back out. Pages of 16 slots with key sizes
+    in steps of 8 and value sizes in steps of 16 take the matrix-core kernel in bfloat16 (fewer heads than 16, exactly
+    16 and more), the others the kernel for any sizes."""
     ops, ref = hip_ops(dtype), TorchOps("cpu", DT[dtype])
     g = torch.Generator().manual_seed(C)
-    ps, n_pages = 8, 12
+    ps, n_pages = (16, 12) if C % 16 == 0 else (8, 12)
     tables = [[5, 2, 9, 0, 0, 0], [7, 1, 3, 11, 4, 0]]
     cols = Hq * (D + R) + C + R + 5
     gain = 1 + 0.2 * torch.randn(C, generator=g)
     freqs = (50.0 ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64) / max(dims, 1))).float()
     w_in = (torch.randn(Hq, C, D, generator=g) / D ** 0.5).to(DT[dtype])
     w_out = (torch.randn(Hq, V, C, generator=g) / C ** 0.5).to(DT[dtype])
-    planes = [torch.full((n_pages, ps * (C + R)), float("nan"), dtype=DT[dtype]) for _ in range(2)]
+    planes = [torch.full((n_pages, ps * (2 * C + R)), float("nan"), dtype=DT[dtype]) for _ in range(2)]
     planes[0] = planes[0].cuda()
     for seq_rows in ([(0, 0, 19)], [(0, 0, 21), (21, 19, 17)]):
         n = sum(r[2] for r in seq_rows)
@@ -152,7 +155,7 @@ def test_attention_over_a_latent(dtype, Hq, D, R, V, C, dims):
             q, q_plain = o.latent_prepare(mv(proj)[:, 5:], 0, Hq * (D + R), b.positions, b.write_slots["g"], plane, Hq, D, R, C, ps,
                                           mv(gain), mv(freqs), dims, 1e-5)
             o.heads_linear(q_plain, mv(w_in), q, C + R)
-            mixed = o.paged_attention_kv(q, plane, b, "g", Hq, 1, C + R, C, ps, 0, 0.3 / C ** 0.5, latent=True)
+            mixed = o.latent_attention(q, plane, b, "g", Hq, C + R, C, ps, 0.3 / C ** 0.5)
             out = torch.zeros(n, Hq * V + 2, dtype=DT[dtype], device=dev)
             o.heads_linear(mixed, mv(w_out), out, V, 2)
             res.append((q, mixed, out))

@@ -252,22 +252,21 @@ class TorchOps:
             c = proj[:, c_off:c_off + C].float()
             c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * gain
             key = torch.cat((c, turned(proj[:, c_off + C:c_off + C + R].float())), dim=-1).to(plane.dtype)
-            pages = plane.view(plane.shape[0], page_size, C + R)
-            pages[write_slots.long() // page_size, write_slots.long() % page_size] = key
+            pages = plane.view(plane.shape[0], -1)
+            page, off = write_slots.long() // page_size, write_slots.long() % page_size
+            pages[:, :page_size * (C + R)].view(-1, page_size, C + R)[page, off] = key
+            pages[:, page_size * (C + R):].view(-1, C, page_size)[page, :, off] = key[:, :C]
         return q.view(n, H * (C + R)), q_plain
 
     def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
-                           scale=None, sink=False, gate=None, latent=False):
+                           scale=None, sink=False, gate=None):
         n = q.shape[0]
         H, G, kd, vd = n_heads, n_kv_heads, key_dim, value_dim
         scale = scale if scale is not None else kd ** -0.5
         tables = batch.block_tables[group]
         pages = plane.view(plane.shape[0], -1)
-        if latent:
-            keys = pages.view(-1, 1, page_size, kd)
-        else:
-            keys = pages[:, :G * page_size * kd].view(-1, G, page_size, kd)
-            vals = pages[:, G * page_size * kd:].view(-1, G, vd, page_size)
+        keys = pages[:, :G * page_size * kd].view(-1, G, page_size, kd)
+        vals = pages[:, G * page_size * kd:].view(-1, G, vd, page_size)
         out = torch.zeros(n, H * vd, dtype=torch.float32, device=q.device)
         pos, seq = batch.positions.tolist(), batch.row_seq.tolist()
         for r in range(n):
@@ -275,7 +274,7 @@ class TorchOps:
             js = torch.arange(max(0, p - window + 1) if window > 0 else 0, p + 1)
             pg = tables[seq[r]].long()[js // page_size]
             k = keys[pg, :, js % page_size].float()          # [keys, G, kd]
-            v = k[..., :vd] if latent else vals[pg, :, :, js % page_size].float()       # [keys, G, vd]
+            v = vals[pg, :, :, js % page_size].float()       # [keys, G, vd]
             qr = q[r].float().view(H, kd)
             for h in range(H):
                 sc = (k[:, h // (H // G)] @ qr[h]) * scale
@@ -288,6 +287,9 @@ class TorchOps:
                     o = o * torch.sigmoid(gate[r, h].float())
                 out[r, h * vd:(h + 1) * vd] = o
         return out.to(q.dtype)
+
+    def latent_attention(self, q, plane, batch, group, n_heads, key_dim, value_dim, page_size, scale):
+        return self.paged_attention_kv(q, plane, batch, group, n_heads, 1, key_dim, value_dim, page_size, 0, scale)
 
     # ---- a residual stream in 32-bit, norm before the sublayer ------------------------------------------------
     def layernorm32(self, x32, gain, bias, eps):

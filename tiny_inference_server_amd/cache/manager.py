@@ -80,7 +80,6 @@ class GroupSpec:
     head_dim: int
     window: int                      # 0: every position stays readable
     value_dim: int = 0               # channels of a value where they differ from head_dim (0: the same)
-    keys_only: bool = False          # a page holds keys alone (the values are part of them)
     keys: List[str] = field(default_factory=list)    # cache keys of the users, in plane order
 
 
@@ -100,11 +99,7 @@ class PageGroup:
             # [plane][page][key or value][kv head][slot in page][head size]; within a page and head the values
             # lie transposed, [head size][slot]. Zeroed once, as the reference does (block_table.py:40), though no
             # kernel needs it: slots that a row may not see are read, but replaced before any arithmetic
-            if spec.keys_only:
-                # keys [kv head][slot][head size] and nothing else
-                self.storage = torch.zeros((len(spec.keys), n_pages, spec.n_kv_heads * page_size * spec.head_dim),
-                                           dtype=dtype, device=device)
-            elif spec.value_dim and spec.value_dim != spec.head_dim:
+            if spec.value_dim and spec.value_dim != spec.head_dim:
                 # keys [kv head][slot][head size] of all heads, then values [kv head][value size][slot]: one line a page
                 self.storage = torch.zeros((len(spec.keys), n_pages,
                                             spec.n_kv_heads * page_size * (spec.head_dim + spec.value_dim)),
@@ -189,19 +184,18 @@ class CacheManager:
         n_slots = max_requests + (1 if spare_positions > 0 else 0)
         n_pages = n_pages + self._spare_pages
         self.dtype, self.device = dtype, device
-        specs: Dict[Tuple[int, int, int, int, bool], GroupSpec] = {}
+        specs: Dict[Tuple[int, int, int, int], GroupSpec] = {}
         self.group_of: Dict[str, str] = {}
         self.states: Dict[str, Optional[torch.Tensor]] = {}
         self._state_needs: Dict[str, StateNeed] = {}
         for key, need in needs.items():
             if isinstance(need, PagedKvNeed):
-                only = bool(need.values_in_keys)
-                vdim = need.value_dim if need.value_dim and need.value_dim != need.head_dim and not only else 0
-                geom = (need.n_kv_heads, need.head_dim, need.window, vdim, only)
+                vdim = need.value_dim if need.value_dim and need.value_dim != need.head_dim else 0
+                geom = (need.n_kv_heads, need.head_dim, need.window, vdim)
                 if geom not in specs:
-                    name = (("k" if only else "kv") + f"{need.n_kv_heads}x{need.head_dim}" + (f"v{vdim}" if vdim else "") +
+                    name = (f"kv{need.n_kv_heads}x{need.head_dim}" + (f"v{vdim}" if vdim else "") +
                             (f"w{need.window}" if need.window else ""))
-                    specs[geom] = GroupSpec(name, need.n_kv_heads, need.head_dim, need.window, vdim, only)
+                    specs[geom] = GroupSpec(name, need.n_kv_heads, need.head_dim, need.window, vdim)
                 specs[geom].keys.append(key)
                 self.group_of[key] = specs[geom].name
             elif isinstance(need, StateNeed):
@@ -295,14 +289,13 @@ class CacheManager:
         """Bytes that one more page costs: every group gets as many pages as every other, and a page of a group has
         a plane for each of the group's cache users (the reference's one geometry: block_table.py:34-38)."""
         elem = torch.empty(0, dtype=dtype).element_size()
-        return sum(need.n_kv_heads * (need.head_dim + (0 if need.values_in_keys else need.value_dim or need.head_dim))
-                   * page_size * elem for need in needs.values() if isinstance(need, PagedKvNeed))
+        return sum(need.n_kv_heads * (need.head_dim + (need.value_dim or need.head_dim)) * page_size * elem
+                   for need in needs.values() if isinstance(need, PagedKvNeed))
 
     def bytes_per_position(self) -> int:
         """Bytes of keys and values that one position of one request takes, over all groups and planes."""
         elem = torch.empty(0, dtype=self.dtype).element_size()
-        return sum(len(g.spec.keys) * g.spec.n_kv_heads *
-                   (g.spec.head_dim + (0 if g.spec.keys_only else g.spec.value_dim or g.spec.head_dim)) * elem
+        return sum(len(g.spec.keys) * g.spec.n_kv_heads * (g.spec.head_dim + (g.spec.value_dim or g.spec.head_dim)) * elem
                    for g in self.groups.values())
 
     def free_pages(self) -> Dict[str, int]:

@@ -6,7 +6,7 @@
 //
 // A page of `page_size` slots holds, for each key/value head, the keys as [slot][key size] and then, after the keys
 // of all heads, the values transposed as [value size][slot]. With equal sizes that is the layout the other attention
-// kernels read. Pages of a latent hold keys only; the values are the keys' first channels. The row at position p sees
+// kernels read. The row at position p sees
 // the keys at [max(0, p - window + 1), p] (window 0: all), found through the request's block table; keys outside are
 // never read, so what a reused page holds cannot reach a result.
 // Norms, angles, scores, the softmax and the weighted sum are 32-bit; `T` is the type of queries and pages.
@@ -111,11 +111,13 @@ __global__ __launch_bounds__(TIS_WAVE) void attention_prepare_kernel(
 }
 
 // The same step where all heads share one latent as keys and values. grid (rows, H + 1), one wave each.
-// Unit u < H, a query head: the head's R rotated channels (32-bit, at q_off + u * (D + R) + D of proj) are turned by
+// (A latent's pages are those of one key/value head with keys of C + R and values of C channels: the latent is kept
+// twice, as the first channels of its key and transposed as its value.) Unit u < H, a query head: the head's R rotated channels (32-bit, at q_off + u * (D + R) + D of proj) are turned by
 // the row's position and written to q_out[u * (C + R) + C ...]; its D unrotated channels go, in the compute type, to
 // q_plain[u * D ...] (for the product that takes them into the latent's space, whose result belongs to
 // q_out[u * (C + R) ...]). Unit H: the row's latent, C channels at c_off, RMS-normed with `gain`, then the R channels
-// of the shared rotated key, turned alike; both go into the row's slot of a page of [slot][C + R] keys.
+// of the shared rotated key, turned alike; both go into the row's slot of the page's keys, and the latent also into
+// its values.
 template <typename T>
 __global__ __launch_bounds__(TIS_WAVE) void latent_prepare_kernel(
     const float* __restrict__ proj, long ldp, int q_off, int c_off, const int* __restrict__ positions,
@@ -135,13 +137,19 @@ __global__ __launch_bounds__(TIS_WAVE) void latent_prepare_kernel(
   } else {
     if (!write_slots) return;
     const int ws = write_slots[r];
-    T* key = plane + ((long)(ws / page_size) * page_size + ws % page_size) * (C + R);
+    T* page = plane + (long)(ws / page_size) * page_size * (2 * C + R);
+    T* key = page + (long)(ws % page_size) * (C + R);
+    T* val = page + (long)page_size * (C + R) + ws % page_size;
     src = proj + r * ldp + c_off;
     float ss = 0.f;
     for (int e = lane; e < C; e += TIS_WAVE) ss += src[e] * src[e];
     ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)C + eps);
-    for (int e = lane; e < C; e += TIS_WAVE) key[e] = from_f<T>(src[e] * inv * gain[e]);
+    for (int e = lane; e < C; e += TIS_WAVE) {
+      const T v = from_f<T>(src[e] * inv * gain[e]);
+      key[e] = v;
+      val[(long)e * page_size] = v;
+    }
     src += C;
     dst = key + C;
   }
@@ -163,13 +171,11 @@ __global__ __launch_bounds__(TIS_WAVE) void latent_prepare_kernel(
 // One workgroup per (row, query head). Keys are walked in chunks of AW_CHUNK with a running maximum; the order of
 // every sum depends on the row's own position and window only. sink: the softmax's denominator also holds a key of
 // score 0 that has no value. gate (nullable): the head's result is multiplied by sigmoid(gate[row * ldg + head]).
-// latent: a page holds keys only, [slot][KD], and a key's first VD channels are its value.
 template <typename T>
 __global__ __launch_bounds__(AW_THREADS) void attention_window_kernel(
     const T* __restrict__ q, long ldq, const T* __restrict__ plane, const int* __restrict__ block_tables, int bt_ld,
     const int* __restrict__ row_seq, const int* __restrict__ positions, T* __restrict__ out, long ldo, int group_size,
-    int G, int KD, int VD, int page_size, int window, float scale, int sink, const float* __restrict__ gate, long ldg,
-    int latent) {
+    int G, int KD, int VD, int page_size, int window, float scale, int sink, const float* __restrict__ gate, long ldg) {
   __shared__ float qs[AW_MAX_DIM];
   __shared__ float sc[AW_CHUNK];
   __shared__ float red[16];
@@ -182,10 +188,9 @@ __global__ __launch_bounds__(AW_THREADS) void attention_window_kernel(
   const int end = pos + 1;
   for (int d = t; d < KD; d += AW_THREADS) qs[d] = to_f(q[r * ldq + (long)h * KD + d]) * scale;
   __syncthreads();
-  const long page_stride = latent ? (long)G * page_size * KD : (long)G * page_size * (KD + VD);
+  const long page_stride = (long)G * page_size * (KD + VD);
   const long k_off = (long)g * page_size * KD;
-  const long v_off = latent ? k_off : (long)G * page_size * KD + (long)g * VD * page_size;
-  const long v_slot = latent ? KD : 1, v_chan = latent ? 1 : page_size;
+  const long v_off = (long)G * page_size * KD + (long)g * VD * page_size;
   // a thread owns `per` value channels, width apart; the threads that share a channel take every n-th key
   const int per = (VD + AW_THREADS - 1) / AW_THREADS;
   const int width = (VD + per - 1) / per;
@@ -224,11 +229,11 @@ __global__ __launch_bounds__(AW_THREADS) void attention_window_kernel(
     if (pv) {
       for (int i = part; i < n; i += lanes_per_key) {
         const int j = c0 + i;
-        const T* vp = plane + (long)bt[j / page_size] * page_stride + v_off + (long)(j % page_size) * v_slot;
+        const T* vp = plane + (long)bt[j / page_size] * page_stride + v_off + (j % page_size);
         const float p = sc[i];
 #pragma unroll
         for (int u = 0; u < AW_PER; ++u)
-          if (u < per && d + u * width < VD) acc[u] += p * to_f(vp[(long)(d + u * width) * v_chan]);
+          if (u < per && d + u * width < VD) acc[u] += p * to_f(vp[(long)(d + u * width) * page_size]);
       }
     }
     __syncthreads();
@@ -297,20 +302,19 @@ TIS_EXPORT int tis_latent_prepare(int dtype, const float* proj, long ldp, int q_
 TIS_EXPORT int tis_attention_window(int dtype, const void* q, long ldq, const void* plane, const int* block_tables,
                                     int bt_ld, const int* row_seq, const int* positions, void* out, long ldo, int rows,
                                     int H, int G, int KD, int VD, int page_size, int window, float scale, int sink,
-                                    const float* gate, long ldg, int latent, hipStream_t stream) {
+                                    const float* gate, long ldg, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || H < 1 || G < 1 || H % G || page_size < 1 || window < 0 || H > 65535)
     return tis_fail("attention_window: bad size rows=%d heads=%d kv_heads=%d page=%d window=%d", rows, H, G, page_size, window);
   if (KD < 1 || KD > AW_MAX_DIM || VD < 1 || VD > AW_MAX_DIM)
     return tis_fail("attention_window: key size %d or value size %d is outside 1..%d", KD, VD, AW_MAX_DIM);
-  if (latent && VD > KD) return tis_fail("attention_window: a latent's value (%d) is part of its key (%d)", VD, KD);
   dim3 grid(rows, H);
   if (dtype == TIS_F32)
     attention_window_kernel<float><<<grid, AW_THREADS, 0, stream>>>((const float*)q, ldq, (const float*)plane, block_tables,
-        bt_ld, row_seq, positions, (float*)out, ldo, H / G, G, KD, VD, page_size, window, scale, sink, gate, ldg, latent);
+        bt_ld, row_seq, positions, (float*)out, ldo, H / G, G, KD, VD, page_size, window, scale, sink, gate, ldg);
   else if (dtype == TIS_BF16)
     attention_window_kernel<bf16><<<grid, AW_THREADS, 0, stream>>>((const bf16*)q, ldq, (const bf16*)plane, block_tables,
-        bt_ld, row_seq, positions, (bf16*)out, ldo, H / G, G, KD, VD, page_size, window, scale, sink, gate, ldg, latent);
+        bt_ld, row_seq, positions, (bf16*)out, ldo, H / G, G, KD, VD, page_size, window, scale, sink, gate, ldg);
   else
     return tis_fail("unknown dtype code %d", dtype);
   return tis_launch_status("attention_window");

@@ -44,6 +44,7 @@ SOURCES: Dict[str, str] = {
     "attention_window": "attention_window.hip",
     "state_scan": "state_scan.hip",
     "experts": "experts.hip",
+    "attention_latent": "attention_latent.hip",
 }
 HEADERS = ["common.h", "attention_mfma.h"]
 # what a library links beyond the HIP runtime
@@ -80,6 +81,8 @@ def _hipcc() -> str:
 # libraries compiled once per value of a macro: name -> (macro, values that build() makes without being asked)
 VARIANTS: Dict[str, tuple] = {
     "attention_mfma": ("TIS_HD", (32, 48, 64, 128, 256)),
+    # keys' channels * 10000 + values' channels of a latent (others are built when a model first asks for them)
+    "attention_latent": ("TIS_LATENT", (5760512,)),
 }
 
 

@@ -119,7 +119,10 @@ _SIGNATURES["attention_window"] = ("tis_attention_window", {
     "tis_attention_prepare": [_I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _F, _I,
                               _I, _I, _I, _I, _I, _I, _P],
     "tis_latent_prepare": [_I, _P, _L, _I, _I, _P, _P, _P, _P, _L, _P, _L, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P],
-    "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _I, _P],
+    "tis_attention_window": [_I, _P, _L, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _P],
+})
+_SIGNATURES["attention_latent"] = ("tis_attention_latent", {
+    "tis_attention_latent": [_P, _L, _P, _P, _I, _P, _P, _P, _I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
 })
 _SIGNATURES["experts"] = ("tis_experts", {
     "tis_route_topk": [_P, _L, _P, _F, _I, _I, _I, _P, _P, _P],
@@ -400,6 +403,18 @@ def planned_beside_tiles(seq_rows, items, tiles, tile_steps, n_heads: int, n_kv_
         return None
     return decode_items(singles, n_heads, n_kv_heads, head_dim, window=window, units=units, table_lines=lines,
                         all_rows=all_rows, share=min(1.0, _ATTN_PLANNED_WAVES_BESIDE_TILES / n_kv_heads))
+
+
+def latent_items(seq_rows, n_heads: int):
+    """(first row, rows) of every item of the latent-attention kernel: 16 columns an item, a column a (row, head) pair,
+    so 16 // heads consecutive rows of one request where there are fewer than 16 heads, a single row otherwise."""
+    per = max(1, 16 // n_heads)
+    rows = np.asarray(seq_rows, dtype=np.int64).reshape(-1, 3)
+    first, n = rows[:, 0], rows[:, 2]
+    k = -(-n // per)
+    r = (np.arange(int(k.sum())) - np.repeat(np.cumsum(k) - k, k)) * per
+    counts = np.minimum(per, np.repeat(n, k) - r)
+    return np.stack((np.repeat(first, k) + r, counts), axis=1).astype(np.int32)
 
 
 class AttentionLaunch(NamedTuple):
@@ -1343,8 +1358,9 @@ class HipOps:
         one rotated key part (rot_dim). Returns (q [rows, heads * (rank + rot_dim)] with every head's rotated part in
         place behind `rank` columns that the caller fills, q_plain [rows, heads * dim]: the unrotated parts), both in
         the compute type. The latent, RMS-normed with `gain`, and the rotated key part go into the pages at
-        write_slots as keys of rank + rot_dim channels. Rotation: interleaved pairs of the first rot_dims channels
-        of the rotated parts, angle = position * freqs[pair]."""
+        write_slots as keys of rank + rot_dim channels, and the latent once more as the key's value (pages of one
+        key/value head with keys of rank + rot_dim and values of rank channels). Rotation: interleaved pairs of the
+        first rot_dims channels of the rotated parts, angle = position * freqs[pair]."""
         n = proj.shape[0]
         self._f32_rows(proj, "latent_prepare projections", n, max(q_off + n_heads * (dim + rot_dim), c_off + rank + rot_dim))
         self._index(positions, "positions", n)
@@ -1353,7 +1369,7 @@ class HipOps:
             self._f32(freqs, "rotary frequencies", rot_dims // 2)
         if write_cache:
             self._index(write_slots, "write_slots", n)
-            self._check_latent_plane(plane, rank + rot_dim, page_size)
+            self._check_kv_plane(plane, 1, rank + rot_dim, rank, page_size)
         q = self.empty(n, n_heads * (rank + rot_dim))
         q_plain = self.empty(n, n_heads * max(dim, 1))
         self._lazy("attention_window").tis_latent_prepare(
@@ -1363,25 +1379,72 @@ class HipOps:
             self._stream())
         return q, q_plain
 
-    def _check_latent_plane(self, plane, key_dim, page_size):
-        self._check(plane, "cache plane")
-        if not plane.is_contiguous() or plane.shape[0] < 1 or plane.numel() != plane.shape[0] * page_size * key_dim:
-            raise KernelError(f"cache plane {tuple(plane.shape)} does not hold pages of {page_size} slots x {key_dim}")
+    def plan_latent(self, n_heads: int, seq_rows, add):
+        """Host planning for attention over a latent: the items of the matrix-core kernel for a step's rows, (first row,
+        rows) each, as many consecutive rows of one request as 16 columns hold heads. Steps of single rows need no list."""
+        if self.dtype != torch.bfloat16 or all(n <= 1 for _, _, n in seq_rows):
+            return {}
+        items = latent_items(seq_rows, n_heads)
+        return {("latent_items", n_heads): (add(items), len(items))}
 
-    def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
-                           scale=None, sink=False, gate=None, latent=False):
-        """Attention of the rows in `batch` over pages whose keys have key_dim and whose values value_dim channels:
-        [rows, heads*value_dim]. sink: the softmax's denominator also counts a key of score 0 that has no value.
-        gate: [rows, heads] 32-bit (a strided view is fine); head h's result is multiplied by sigmoid(gate[:, h]).
-        latent: the pages hold keys only and a key's first value_dim channels are its value (one key/value head)."""
+    def latent_attention(self, q, plane, batch, group, n_heads, key_dim, value_dim, page_size, scale):
+        """Attention of the rows in `batch` over the pages of a latent: one key/value head, keys of key_dim channels
+        whose first value_dim are also kept as values. q: [rows, heads * key_dim]; the result [rows, heads * value_dim].
+        bfloat16 with pages of 16 slots, key sizes in steps of 8 and value sizes in steps of 16 run on the matrix cores
+        (a library per pair of sizes, compiled when first asked for); anything else on the kernel for any sizes."""
         _rows_view(self._check(q, "q"), "q")
         n = q.shape[0]
-        if latent:
-            if n_kv_heads != 1 or value_dim > key_dim:
-                raise KernelError(f"attention over a latent: one key/value head, value {value_dim} <= key {key_dim}")
-            self._check_latent_plane(plane, key_dim, page_size)
-        else:
-            self._check_kv_plane(plane, n_kv_heads, key_dim, value_dim, page_size)
+        if not (self.dtype == torch.bfloat16 and page_size == 16 and key_dim % 8 == 0 and value_dim % 16 == 0
+                and value_dim <= key_dim < 10000 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0):
+            return self.paged_attention_kv(q, plane, batch, group, n_heads, 1, key_dim, value_dim, page_size, 0, scale)
+        self._check_kv_plane(plane, 1, key_dim, value_dim, page_size)
+        if q.shape[1] != n_heads * key_dim:
+            raise KernelError(f"attention: q width {q.shape[1]} is not heads {n_heads} x key size {key_dim}")
+        tables = batch.block_tables[group]
+        self._check(tables, "block tables", torch.int32)
+        if tables.dim() != 2 or tables.stride(1) != 1:
+            raise KernelError(f"attention: block tables {tuple(tables.shape)} must be 2-d")
+        self._index(batch.positions, "positions", n)
+        self._index(batch.row_seq, "row_seq", n)
+        if batch.max_kv_len > tables.shape[1] * page_size:
+            raise KernelError(f"attention: a row sees {batch.max_kv_len} keys but block tables cover "
+                              f"{tables.shape[1] * page_size}")
+        out = self.empty(n, n_heads * value_dim)
+        if n == 0:
+            return out
+        items, n_items = None, n
+        if batch.max_seq_rows > 1:
+            plan = batch.extras.get(("latent_items", n_heads))
+            if plan is None:        # a caller that did not plan (a kernel test)
+                host = latent_items(batch.seq_rows, n_heads)
+                plan = (torch.from_numpy(host).reshape(-1).to(self.device), len(host))
+            items, n_items = plan[0].reshape(-1), plan[1]
+            if items.numel() < 2 * n_items or items.dtype != torch.int32 or not items.is_contiguous():
+                raise KernelError(f"attention: a list of {items.numel()} integers for {n_items} items")
+        # enough waves to fill the chip: a request's keys are cut where its items alone would leave most units idle
+        waves = n_items * -(-n_heads // 16)
+        steps = -(-batch.max_kv_len // 32)
+        most = max(1, (self._workspace.numel() // (n * n_heads * (value_dim + 2))))
+        n_splits = int(max(1, min(-(-2 * self.units // waves), steps // 4, 64, most)))
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o = self._workspace
+            part_ml = self._workspace[n * n_heads * n_splits * value_dim:]
+        lib = self._lazy(f"attention_latent@{key_dim * 10000 + value_dim}")
+        lib.tis_attention_latent(_ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
+                                 _ptr(batch.positions), _ptr(items), n_items, _ptr(out), out.stride(0), _ptr(part_o),
+                                 _ptr(part_ml), n, n_heads, key_dim, value_dim, page_size, float(scale), n_splits,
+                                 self._stream())
+        return out
+
+    def paged_attention_kv(self, q, plane, batch, group, n_heads, n_kv_heads, key_dim, value_dim, page_size, window=0,
+                           scale=None, sink=False, gate=None):
+        """Attention of the rows in `batch` over pages whose keys have key_dim and whose values value_dim channels:
+        [rows, heads*value_dim]. sink: the softmax's denominator also counts a key of score 0 that has no value.
+        gate: [rows, heads] 32-bit (a strided view is fine); head h's result is multiplied by sigmoid(gate[:, h])."""
+        _rows_view(self._check(q, "q"), "q")
+        n = q.shape[0]
+        self._check_kv_plane(plane, n_kv_heads, key_dim, value_dim, page_size)
         if q.shape[1] != n_heads * key_dim:
             raise KernelError(f"attention: q width {q.shape[1]} is not heads {n_heads} x key size {key_dim}")
         if gate is not None:
@@ -1400,7 +1463,7 @@ class HipOps:
             self.code, _ptr(q), q.stride(0), _ptr(plane), _ptr(tables), tables.stride(0), _ptr(batch.row_seq),
             _ptr(batch.positions), _ptr(out), out.stride(0), n, n_heads, n_kv_heads, key_dim, value_dim, page_size,
             int(window), float(scale if scale is not None else key_dim ** -0.5), 1 if sink else 0, _ptr(gate),
-            gate.stride(0) if gate is not None else 0, 1 if latent else 0, self._stream())
+            gate.stride(0) if gate is not None else 0, self._stream())
         return out
 
     # ---- recurrent mixers with a matrix state per head ---------------------------------------------------

@@ -274,7 +274,8 @@ class LatentAttention:
     rotation in interleaved pairs of the first rot_dims channels of the rotated parts by position * base^(-2i/rot_dims);
     causal softmax; out = heads . Wo^T.
 
-    Only c and the rotated key part are kept, as one key of rank + rot_dim channels per position. The products with
+    Only c and the rotated key part are kept, as one key of rank + rot_dim channels per position whose value is c
+    again (transposed, as the attention kernels read values). The products with
     Wuk and Wuv are moved to the query's side of the sums: q_plain . (Wuk[h] c) = (Wuk[h]^T q_plain) . c, so a row's
     query becomes [Wuk[h]^T q_plain | q_rot] against the key [c | k_rot]; and sum_j p_j Wuv[h] c_j = Wuv[h] sum_j p_j c_j,
     so the attention's values are the latents themselves and Wuv[h] is applied to the result.
@@ -293,7 +294,7 @@ class LatentAttention:
 
     @classmethod
     def cache_need(cls, params):
-        return PagedKvNeed(1, params["rank"] + params["rot_dim"], 0, value_dim=params["rank"], values_in_keys=True)
+        return PagedKvNeed(1, params["rank"] + params["rot_dim"], 0, value_dim=params["rank"])
 
     def __init__(self, spec, tensors, ops):
         from .base import to_gain
@@ -314,6 +315,13 @@ class LatentAttention:
         self.w_uv = to_compute(ops, tensors.of(spec, "uv").view(self.H, self.V, self.C))
         self.w_o = to_compute(ops, tensors.of(spec, "o"))
 
+    # the matrix-core kernel's items, where a step brings portions
+    def plan_key(self):
+        return ("latent", self.H) if hasattr(self.ops, "plan_latent") else None
+
+    def plan_rows(self, seq_rows, add, mode=None):
+        return self.ops.plan_latent(self.H, seq_rows, add)
+
     def core(self, x, ctx):
         ops, b = self.ops, ctx.batch
         H, D, R, V, C = self.H, self.D, self.R, self.V, self.C
@@ -321,7 +329,7 @@ class LatentAttention:
         q, q_plain = ops.latent_prepare(proj, 0, self.c_at, b.positions, b.write_slots[ctx.group], ctx.plane, H, D, R, C,
                                         ctx.page_size, self.c_gain, self.freqs, self.rot_dims, self.eps, ctx.writes_cache)
         ops.heads_linear(q_plain, self.w_uk_t, q, C + R)
-        mixed = ops.paged_attention_kv(q, ctx.plane, b, ctx.group, H, 1, C + R, C, ctx.page_size, 0, self.scale, latent=True)
+        mixed = ops.latent_attention(q, ctx.plane, b, ctx.group, H, C + R, C, ctx.page_size, self.scale)
         return ops.heads_linear(mixed, self.w_uv, ops.empty(mixed.shape[0], H * V), V)
 
     def forward32(self, x, ctx):

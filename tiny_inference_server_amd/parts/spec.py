@@ -84,13 +84,11 @@ class ModelSpec:
 @dataclass(frozen=True)
 class PagedKvNeed:
     """Keys and values of every position (window 0) or of the last `window` positions. value_dim: channels of a
-    value where they differ from a key's head_dim (0: the same). values_in_keys: nothing is kept beside the keys (a
-    shared latent whose first channels are the values); value_dim then only says how many."""
+    value where they differ from a key's head_dim (0: the same)."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
     value_dim: int = 0
-    values_in_keys: bool = False
 
 
 @dataclass(frozen=True)
