@@ -160,37 +160,78 @@ __global__ __launch_bounds__(256) void grouped_plain_kernel(const TA* __restrict
   }
 }
 
-// bfloat16 on the matrix cores: a wave owns 16 entries x 16 columns, four waves a workgroup side by side in N. A
-// matrix row and an input row are the two operands of v_mfma_f32_16x16x32_bf16 straight from memory, 16 bytes a lane
-// (rows 16-byte aligned, K a multiple of 8). Each result is one wave's sum over K in steps of 32.
-template <typename TO>
+// bfloat16 on the matrix cores. A workgroup of four waves, WM x WN of them, owns 16 RM WM entries x 16 RN WN columns; a
+// wave owns RM x RN tiles of 16 x 16. A matrix row and an input row are the two operands of v_mfma_f32_16x16x32_bf16
+// straight from memory, 16 bytes a lane (rows 16-byte aligned, K a multiple of 8); a wave's RM + RN loads of a step feed
+// RM RN products, and what the waves of a workgroup share meets in the caches. Each result is one wave's sum over K in
+// steps of 32. Two shapes are built: 16 entries x 64 columns for groups of a few rows (decoded tokens: the job is to
+// stream the matrices once), 64 x 128 for groups of many.
+template <typename TO, int WM, int WN, int RM, int RN>
 __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                            TO* __restrict__ C, GroupedArgs p) {
-  const int g = blockIdx.z, m0 = blockIdx.y * 16, t = threadIdx.x, lane = t % 64, wave = t / 64;
-  const int n0 = blockIdx.x * 64 + wave * 16;
+  static_assert(WM * WN == 4, "four waves a workgroup");
+  const int g = blockIdx.z, t = threadIdx.x, lane = t % 64, wave = t / 64;
+  const int m0 = blockIdx.y * (16 * RM * WM) + (wave / WN) * (16 * RM);
+  const int n0 = blockIdx.x * (16 * RN * WN) + (wave % WN) * (16 * RN);
   const int count = p.lists ? p.counts[g] : p.rows;
   if (m0 >= count || n0 >= p.N) return;
   const int c16 = lane & 15, kg = lane >> 4;
-  const int mine = m0 + c16 < count ? (p.lists ? p.lists[(long)g * p.line + m0 + c16] : m0 + c16) : -1;
-  const bf16* arow = A + (long)(mine < 0 ? 0 : mine / p.a_div) * p.lda + (long)g * p.a_group + kg * 8;
-  const bool w_ok = n0 + c16 < p.N;
-  const bf16* wrow = W + ((long)g * p.N + (w_ok ? n0 + c16 : 0)) * p.K + kg * 8;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < p.K; k0 += 32) {
-    const bool k_ok = k0 + kg * 8 < p.K;
-    const bf16x8 wv = (w_ok && k_ok) ? *reinterpret_cast<const bf16x8*>(wrow + k0) : zero;
-    const bf16x8 av = (mine >= 0 && k_ok) ? *reinterpret_cast<const bf16x8*>(arow + k0) : zero;
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc, 0, 0, 0);
-  }
-  // the lane holds the columns n0 + 4 kg + i of entry c16
-  if (mine < 0) return;
+  int mine[RM];
+  const bf16* arow[RM];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int n = n0 + 4 * kg + i;
-    if (n >= p.N) continue;
-    const float v = p.act == 1 ? gelu_erf_f(acc[i]) : acc[i];
-    C[(long)mine * p.ldc + (long)g * p.c_group + n] = from_f<TO>(v);
+  for (int i = 0; i < RM; ++i) {
+    const int m = m0 + i * 16 + c16;
+    mine[i] = m < count ? (p.lists ? p.lists[(long)g * p.line + m] : m) : -1;
+    arow[i] = A + (long)(mine[i] < 0 ? 0 : mine[i] / p.a_div) * p.lda + (long)g * p.a_group + kg * 8;
+  }
+  bool w_ok[RN];
+  const bf16* wrow[RN];
+#pragma unroll
+  for (int j = 0; j < RN; ++j) {
+    w_ok[j] = n0 + j * 16 + c16 < p.N;
+    wrow[j] = W + ((long)g * p.N + (w_ok[j] ? n0 + j * 16 + c16 : 0)) * p.K + kg * 8;
+  }
+  f32x4 acc[RM][RN];
+#pragma unroll
+  for (int i = 0; i < RM; ++i)
+#pragma unroll
+    for (int j = 0; j < RN; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  // U steps of 32 at a time: all their loads are issued before the first product, so that a wave keeps several
+  // steps' worth of requests in flight (the products of one step take far less time than its operands' way here)
+  constexpr int U = 4;
+  for (int k0 = 0; k0 < p.K; k0 += 32 * U) {
+    bf16x8 av[U][RM], wv[U][RN];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u * 32;
+      const bool k_ok = k + kg * 8 < p.K;
+#pragma unroll
+      for (int i = 0; i < RM; ++i) av[u][i] = (mine[i] >= 0 && k_ok) ? *reinterpret_cast<const bf16x8*>(arow[i] + k) : zero;
+#pragma unroll
+      for (int j = 0; j < RN; ++j) wv[u][j] = (w_ok[j] && k_ok) ? *reinterpret_cast<const bf16x8*>(wrow[j] + k) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < RM; ++i)
+#pragma unroll
+        for (int j = 0; j < RN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u][j], av[u][i], acc[i][j], 0, 0, 0);
+  }
+  // the lane holds, of tile (i, j), the columns n0 + 16 j + 4 kg + e of entry i * 16 + c16
+#pragma unroll
+  for (int i = 0; i < RM; ++i) {
+    if (mine[i] < 0) continue;
+#pragma unroll
+    for (int j = 0; j < RN; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int n = n0 + j * 16 + 4 * kg + e;
+        if (n >= p.N) continue;
+        const float v = p.act == 1 ? gelu_erf_f(acc[i][j][e]) : acc[i][j][e];
+        C[(long)mine[i] * p.ldc + (long)g * p.c_group + n] = from_f<TO>(v);
+      }
   }
 }
 
@@ -244,9 +285,14 @@ TIS_EXPORT int tis_grouped_linear(int in_dtype, int out_dtype, const void* A, lo
   dim3 grid((N + 63) / 64, tiles_m, groups);
   if (in_dtype == TIS_BF16) {
     const bool aligned = K % 8 == 0 && lda % 8 == 0 && a_group % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0;
-    if (aligned) {
-      if (out_dtype == TIS_BF16) grouped_mfma_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (bf16*)C, p);
-      else grouped_mfma_kernel<float><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (float*)C, p);
+    if (aligned && most_rows >= 64 * (lists ? groups : 1)) {
+      // groups of many rows (with lists: if the rows were spread evenly): 64 entries x 128 columns a workgroup
+      dim3 big((N + 127) / 128, (most_rows + 63) / 64, groups);
+      if (out_dtype == TIS_BF16) grouped_mfma_kernel<bf16, 2, 2, 2, 4><<<big, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (bf16*)C, p);
+      else grouped_mfma_kernel<float, 2, 2, 2, 4><<<big, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (float*)C, p);
+    } else if (aligned) {
+      if (out_dtype == TIS_BF16) grouped_mfma_kernel<bf16, 1, 4, 1, 1><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (bf16*)C, p);
+      else grouped_mfma_kernel<float, 1, 4, 1, 1><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (float*)C, p);
     } else {
       if (out_dtype == TIS_BF16) grouped_plain_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (bf16*)C, p);
       else grouped_plain_kernel<bf16, float><<<grid, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (float*)C, p);
