@@ -165,7 +165,7 @@ def test_attention_over_a_latent(dtype, Hq, D, R, V, C, dims):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n,W,F,E,I,top", [(37, 64, 40, 6, 2, 2), (5, 44, 20, 3, 3, 6), (200, 128, 72, 16, 1, 3), (9, 48, 30, 2, 0, 1), (600, 64, 48, 4, 1, 2),
+@pytest.mark.parametrize("n,W,F,E,I,top", [(37, 64, 40, 6, 2, 2), (5, 44, 20, 3, 3, 6), (200, 128, 72, 16, 1, 3), (9, 48, 30, 2, 0, 1), (600, 64, 48, 4, 1, 2), (700, 128, 72, 4, 0, 2),
                                            (4, 32, 8, 0, 3, 2)])
 def test_router_and_experts(dtype, n, W, F, E, I, top):
     ops, ref = hip_ops(dtype), TorchOps("cpu", DT[dtype])

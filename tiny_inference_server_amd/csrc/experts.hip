@@ -235,6 +235,122 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16* __restric
   }
 }
 
+// Groups of many rows: the same product tiled in both directions on v_mfma_f32_32x32x16_bf16 with both operands
+// through LDS, as the tiled product for many rows does it (gemm_tiles.hip: direct loads into LDS one step of 64 ahead,
+// two buffers, a row's eight 16-byte pieces XORed by half the row's number against bank conflicts, the tile computed
+// transposed so that a lane ends up with four consecutive columns). What differs: a tile's rows are list entries, each
+// with an address of its own for reading and for writing, the matrix is the group's, a tile past the group's count
+// leaves at once, and the epilogue may apply the activation. 128 entries x 128 columns, four waves.
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+static __device__ __attribute__((aligned(16))) unsigned char ex_zeros[16];
+
+#pragma clang diagnostic ignored "-Winline-asm"   // M0 in a clobber list: meant
+__device__ __forceinline__ void ex_copy16(const void* lane_src, unsigned lds_addr) {
+  const unsigned base = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_addr);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(lane_src), "s"(base) : "memory", "m0");
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void grouped_tiles_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                            TO* __restrict__ C, GroupedArgs p) {
+  constexpr int BM = 128, BN = 128, WN = 2, BK = 64, PCS = 8, ROWS = BM + BN, WAVES = 4;
+  constexpr int STAGE = ROWS * BK * 2;                  // bytes of a buffer: the entries' rows, then the matrix's
+  constexpr int LPW = ROWS * PCS / 64 / WAVES;          // loads of a step that each wave issues, 8 rows each
+  constexpr int TM = 2, TN = 2;                         // 32 x 32 result tiles of a wave
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * STAGE];
+  const int g = blockIdx.z;
+  const int count = p.lists ? p.counts[g] : p.rows;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  if (m0 >= count) return;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, r32 = lane & 31, h = lane >> 5;
+  const int wm = wave / WN, wn = wave % WN;
+  const unsigned lds0 = (unsigned)(uintptr_t)(const __attribute__((address_space(3))) unsigned char*)lds;
+  const bf16* Wg = W + (long)g * p.N * p.K;
+  auto entry = [&](int m) {                             // the list entry of the tile's row m (the last one again past the count)
+    const int e = min(m0 + m, count - 1);
+    return p.lists ? p.lists[(long)g * p.line + e] : e;
+  };
+  const unsigned char* lane_src[LPW];                   // the lane's piece of its row at K offset 0
+  int lane_piece[LPW];
+#pragma unroll
+  for (int j = 0; j < LPW; ++j) {
+    const int row = (wave * LPW + j) * 8 + (lane >> 3);
+    lane_piece[j] = (lane & 7) ^ ((row >> 1) & 7);
+    const bf16* src = row < BM ? A + (long)(entry(row) / p.a_div) * p.lda + (long)g * p.a_group
+                               : Wg + (long)min(p.N - 1, n0 + row - BM) * p.K;
+    lane_src[j] = (const unsigned char*)src + lane_piece[j] * 16;
+  }
+  auto stage = [&](int k0, int buf) {
+#pragma unroll
+    for (int j = 0; j < LPW; ++j) {
+      const bool inside = k0 + lane_piece[j] * 8 < p.K;
+      ex_copy16(inside ? lane_src[j] + (long)k0 * 2 : ex_zeros, lds0 + buf * STAGE + (wave * LPW + j) * 1024);
+    }
+  };
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  unsigned a_row[TM], b_row[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) a_row[i] = wm * 64 + i * 32 + r32;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) b_row[j] = BM + wn * 64 + j * 32 + r32;
+  const int nk = (p.K + BK - 1) / BK;
+  stage(0, 0);
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");      // this wave's pieces of step kt are in LDS
+    __builtin_amdgcn_s_barrier();                             // ... and everyone's; everyone has read step kt - 1
+    if (kt + 1 < nk) stage((kt + 1) * BK, buf ^ 1);
+    const unsigned char* st = lds + buf * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8 a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        a[i] = *(const bf16x8*)(st + (a_row[i] * PCS + ((2 * ks + h) ^ ((a_row[i] >> 1) & 7))) * 16);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[j] = *(const bf16x8*)(st + (b_row[j] * PCS + ((2 * ks + h) ^ ((b_row[j] >> 1) & 7))) * 16);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
+    }
+  }
+  // accumulator 4 q + e of block (i, j): entry wm * 64 + i * 32 + r32 of the tile, column n0 + wn * 64 + j * 32 + 8 q + 4 h + e
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = wm * 64 + i * 32 + r32;
+    if (m0 + m >= count) continue;
+    TO* dst = C + (long)entry(m) * p.ldc + (long)g * p.c_group;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * 64 + j * 32 + q * 8 + h * 4;
+        if (n >= p.N) continue;               // (N is a multiple of 4: the four columns are inside or outside together)
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = p.act == 1 ? gelu_erf_f(acc[i][j][q * 4 + e]) : acc[i][j][q * 4 + e];
+        if constexpr (sizeof(TO) == 4) {
+          *(f32x4*)(dst + n) = (f32x4){v[0], v[1], v[2], v[3]};
+        } else {
+          bf16x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = static_cast<__bf16>(v[e]);
+          *(bf16x4*)(dst + n) = o;
+        }
+      }
+  }
+}
+
 // out[r] = sum_k weight[r][k] * (y[r * top + k] if ids[r][k] < n_experts else x[r]), in 32-bit
 template <typename T>
 __global__ __launch_bounds__(256) void experts_combine_kernel(const float* __restrict__ y, long ldy, const T* __restrict__ x,
@@ -285,8 +401,17 @@ TIS_EXPORT int tis_grouped_linear(int in_dtype, int out_dtype, const void* A, lo
   dim3 grid((N + 63) / 64, tiles_m, groups);
   if (in_dtype == TIS_BF16) {
     const bool aligned = K % 8 == 0 && lda % 8 == 0 && a_group % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0;
-    if (aligned && most_rows >= 64 * (lists ? groups : 1)) {
-      // groups of many rows (with lists: if the rows were spread evenly): 64 entries x 128 columns a workgroup
+    // what a lane stores four columns at a time must be aligned for it
+    const int oa = out_dtype == TIS_BF16 ? 8 : 16;
+    const bool wide_ok = aligned && N % 4 == 0 && ldc % 4 == 0 && c_group % 4 == 0 && ((uintptr_t)C % oa) == 0 && K >= 64;
+    if (wide_ok && most_rows >= 128 * (lists ? groups : 1)) {
+      // groups of many rows (with lists: if the rows were spread evenly): 128 entries x 128 columns through LDS
+      dim3 big((N + 127) / 128, (most_rows + 127) / 128, groups);
+      if (big.y > 65535) return tis_fail("grouped_linear: %d rows are too many for one call", most_rows);
+      if (out_dtype == TIS_BF16) grouped_tiles_kernel<bf16><<<big, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (bf16*)C, p);
+      else grouped_tiles_kernel<float><<<big, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (float*)C, p);
+    } else if (aligned && most_rows >= 64 * (lists ? groups : 1)) {
+      // 64 entries x 128 columns a workgroup, operands straight from memory
       dim3 big((N + 127) / 128, (most_rows + 63) / 64, groups);
       if (out_dtype == TIS_BF16) grouped_mfma_kernel<bf16, 2, 2, 2, 4><<<big, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (bf16*)C, p);
       else grouped_mfma_kernel<float, 2, 2, 2, 4><<<big, 256, 0, stream>>>((const bf16*)A, (const bf16*)W, (float*)C, p);
