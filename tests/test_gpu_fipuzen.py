@@ -126,7 +126,7 @@ def test_attention_with_bias_sink_query_factor_and_head_gate(dtype, Hq, G, kd, v
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("Hq,D,R,V,C,dims", [(3, 16, 8, 12, 24, 8), (2, 5, 6, 7, 300, 4), (8, 64, 32, 64, 128, 32), (1, 12, 0, 9, 40, 0),
-                                             (20, 24, 16, 8, 48, 16), (16, 128, 64, 128, 512, 64)])
+                                             (20, 24, 16, 8, 48, 16), (16, 128, 64, 128, 512, 64), (70, 8, 8, 16, 32, 8)])
 def test_attention_over_a_latent(dtype, Hq, D, R, V, C, dims):
     """The step before (norm of the latent, rotation, the pages), the product per head into the latent's space, the
     attention whose values are part of its keys, and the product per head back out. Pages of 16 slots with key sizes

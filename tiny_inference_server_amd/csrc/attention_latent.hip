@@ -155,6 +155,130 @@ __global__ __launch_bounds__(64) void latent_mfma_kernel(
   }
 }
 
+// Portions of prompts: a workgroup of four waves takes an item of 64 columns (with fewer than 64 heads, 64 / heads
+// consecutive rows of one request; else a row's heads in blocks of 64), 16 columns a wave. A step's keys and transposed
+// values are copied into LDS once per workgroup and are every wave's MFMA operands from there, so a key is fetched
+// once per 64 columns instead of once per 16. Key rows lie 16 bytes further apart in LDS than in memory, so that the
+// sixteen keys a group of lanes reads at one channel offset fall into different banks.
+static constexpr int TK_STRIDE = KD + 8;                       // elements between two keys in LDS
+static constexpr int TK_BYTES = 32 * TK_STRIDE * 2, TV_BYTES = 2 * VD * PAGE * 2;
+
+__global__ __launch_bounds__(256) void latent_tile_kernel(
+    const bf16* __restrict__ q, long ldq, const bf16* __restrict__ plane, const int* __restrict__ block_tables, int bt_ld,
+    const int* __restrict__ row_seq, const int* __restrict__ positions, const int2* __restrict__ items,
+    bf16* __restrict__ out, long ldo, int H, float scale_log2) {
+  __shared__ __attribute__((aligned(16))) bf16 k_lds[32 * TK_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16 v_lds[2 * VD * PAGE];
+  const int item = blockIdx.x, hb = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c16 = lane & 15, g = lane >> 4;
+  const int row0 = items[item].x, n_rows = items[item].y;
+  const int p_first = positions[row0];
+  const int* bt = block_tables + (long)row_seq[row0] * bt_ld;
+  const int p_last = p_first + n_rows - 1;
+  const int c = wave * 16 + c16;                                // the lane's column among the item's 64
+  const int ro = H >= 64 ? 0 : c / H;
+  const int head = H >= 64 ? hb * 64 + c : c % H;
+  const bool col_ok = ro < n_rows && head < H && (H >= 64 || c < (64 / H) * H);
+  const int col_row = row0 + (col_ok ? ro : 0);
+  const int col_pos = col_ok ? p_first + ro : -1;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  bf16x8 qb[DC];
+#pragma unroll
+  for (int dc = 0; dc < DC; ++dc) {
+    const int d = dc * 32 + g * 8;
+    qb[dc] = (col_ok && d < KD) ? *reinterpret_cast<const bf16x8*>(q + (long)col_row * ldq + (long)head * KD + d) : zero8;
+  }
+  f32x4 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) o[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const long page_stride = (long)PAGE * (KD + VD);
+  const int n_steps = p_last / 32 + 1;
+  constexpr int KP = KD / 8;                                    // 16-byte pieces of a key
+  constexpr int VP = VD * PAGE / 8;                             // ... of a page's values
+
+  for (int s = 0; s < n_steps; ++s) {
+    const int kb = s * 32;
+    const bool ok1 = kb + 16 <= p_last;
+    const bf16* pg0 = plane + (long)bt[kb >> 4] * page_stride;
+    const bf16* pg1 = plane + (long)(ok1 ? bt[(kb >> 4) + 1] : bt[kb >> 4]) * page_stride;
+    __syncthreads();                                            // everyone has read the step before
+    for (int i = tid; i < 32 * KP; i += 256) {
+      const int key = i / KP, piece = i % KP;
+      const bf16* src = (key < 16 ? pg0 : pg1) + (long)(key & 15) * KD + piece * 8;
+      *reinterpret_cast<bf16x8*>(k_lds + key * TK_STRIDE + piece * 8) = *reinterpret_cast<const bf16x8*>(src);
+    }
+    for (int i = tid; i < 2 * VP; i += 256) {
+      const int pgi = i / VP, piece = i % VP;
+      const bf16* src = (pgi ? pg1 : pg0) + (long)PAGE * KD + piece * 8;
+      *reinterpret_cast<bf16x8*>(v_lds + pgi * VD * PAGE + piece * 8) = *reinterpret_cast<const bf16x8*>(src);
+    }
+    __syncthreads();
+    f32x4 st0 = {0.f, 0.f, 0.f, 0.f}, st1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) {
+      const int d = dc * 32 + g * 8;
+      const bf16x8 k0 = d < KD ? *reinterpret_cast<const bf16x8*>(k_lds + c16 * TK_STRIDE + d) : zero8;
+      const bf16x8 k1 = d < KD ? *reinterpret_cast<const bf16x8*>(k_lds + (16 + c16) * TK_STRIDE + d) : zero8;
+      st0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qb[dc], st0, 0, 0, 0);
+      st1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qb[dc], st1, 0, 0, 0);
+    }
+    float sv[8];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key0 = kb + 4 * g + i, key1 = key0 + 16;
+      sv[i] = key0 <= col_pos ? st0[i] * scale_log2 : -INFINITY;
+      sv[4 + i] = (ok1 && key1 <= col_pos) ? st1[i] * scale_log2 : -INFINITY;
+      tmax = fmaxf(tmax, fmaxf(sv[i], sv[4 + i]));
+    }
+    tmax = quad_max(tmax);
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2f(m - m_use);
+    float psum = 0.f;
+    bf16x8 pb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float p = exp2f(sv[e] - m_use);
+      psum += p;
+      pb[e] = static_cast<__bf16>(p);
+    }
+    l = l * alpha + psum;
+    m = m_new;
+    const bool last = kb + 31 > p_last;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int off = (db * 16 + c16) * PAGE + 4 * g;
+      const bf16x4 lo = *reinterpret_cast<const bf16x4*>(v_lds + off);
+      const bf16x4 hi = ok1 ? *reinterpret_cast<const bf16x4*>(v_lds + VD * PAGE + off) : (bf16x4){0, 0, 0, 0};
+      bf16x8 va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      if (last) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (kb + 4 * g + i > p_last) va[i] = static_cast<__bf16>(0.f);
+          if (kb + 16 + 4 * g + i > p_last) va[4 + i] = static_cast<__bf16>(0.f);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, o[db], 0, 0, 0);
+    }
+  }
+  const float lt = quad_sum(l);
+  if (!col_ok) return;
+  const float inv = 1.f / lt;
+  bf16* dst = out + (long)col_row * ldo + (long)head * VD + 4 * g;
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    bf16x4 w;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = static_cast<__bf16>(o[db][i] * inv);
+    *reinterpret_cast<bf16x4*>(dst + db * 16) = w;
+  }
+}
+
 // out[row, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s over a (row, head)'s splits, in a fixed order
 __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
                                                            bf16* __restrict__ out, long ldo, int H, int n_splits) {
@@ -182,6 +306,8 @@ TIS_EXPORT int tis_attention_latent_dims() { return TIS_LATENT; }
 
 // items: (first row, rows) per item, or null where every item is the single row of its own index. part_o / part_ml:
 // [rows][H][n_splits][VD] floats and [rows][H][n_splits] (maximum, sum) pairs, needed where n_splits > 1.
+// n_splits 0: the items are those of the four-wave kernel (64 columns each: 64 / H rows, or a row's heads in blocks of
+// 64), which takes every item's keys whole.
 TIS_EXPORT int tis_attention_latent(const void* q, long ldq, const void* plane, const int* block_tables, int bt_ld,
                                     const int* row_seq, const int* positions, const int* items, int n_items, void* out,
                                     long ldo, float* part_o, float* part_ml, int rows, int H, int key_dim, int value_dim,
@@ -189,11 +315,19 @@ TIS_EXPORT int tis_attention_latent(const void* q, long ldq, const void* plane, 
   if (rows == 0 || n_items == 0) return 0;
   if (key_dim != KD || value_dim != VD) return tis_fail("attention_latent: built for keys of %d and values of %d, called with %d and %d", KD, VD, key_dim, value_dim);
   if (page_size != PAGE) return tis_fail("attention_latent: pages of %d slots (this kernel takes %d)", page_size, PAGE);
-  if (rows < 0 || n_items < 0 || H < 1 || n_splits < 1 || n_splits > 65535 || (H + 15) / 16 > 65535)
+  if (rows < 0 || n_items < 0 || H < 1 || n_splits < 0 || n_splits > 65535 || (H + 15) / 16 > 65535)
     return tis_fail("attention_latent: bad size rows=%d items=%d heads=%d splits=%d", rows, n_items, H, n_splits);
   if (n_splits > 1 && (!part_o || !part_ml)) return tis_fail("attention_latent: %d splits need a workspace", n_splits);
   if ((ldq % 8) || (ldo % 4) || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)plane % 16))
     return tis_fail("attention_latent: q, out and the cache plane must be 16-byte aligned with row strides in steps of 8");
+  if (n_splits == 0) {
+    if (!items) return tis_fail("attention_latent: the four-wave kernel needs its list of items");
+    dim3 tgrid(n_items, (H + 63) / 64);
+    latent_tile_kernel<<<tgrid, 256, 0, stream>>>((const bf16*)q, ldq, (const bf16*)plane, block_tables, bt_ld, row_seq,
+                                                  positions, (const int2*)items, (bf16*)out, ldo, H,
+                                                  scale * 1.4426950408889634f);
+    return tis_launch_status("attention_latent tiles");
+  }
   dim3 grid(n_items, (H + 15) / 16, n_splits);
   latent_mfma_kernel<<<grid, 64, 0, stream>>>((const bf16*)q, ldq, (const bf16*)plane, block_tables, bt_ld, row_seq, positions,
                                              (const int2*)items, (bf16*)out, ldo, part_o, (float2*)part_ml, H,

@@ -405,10 +405,11 @@ def planned_beside_tiles(seq_rows, items, tiles, tile_steps, n_heads: int, n_kv_
                         all_rows=all_rows, share=min(1.0, _ATTN_PLANNED_WAVES_BESIDE_TILES / n_kv_heads))
 
 
-def latent_items(seq_rows, n_heads: int):
-    """(first row, rows) of every item of the latent-attention kernel: 16 columns an item, a column a (row, head) pair,
-    so 16 // heads consecutive rows of one request where there are fewer than 16 heads, a single row otherwise."""
-    per = max(1, 16 // n_heads)
+def latent_items(seq_rows, n_heads: int, columns: int = 64):
+    """(first row, rows) of every item of the latent-attention kernel for portions: `columns` columns an item, a column a
+    (row, head) pair, so columns // heads consecutive rows of one request where there are fewer heads than columns, a
+    single row otherwise."""
+    per = max(1, columns // n_heads)
     rows = np.asarray(seq_rows, dtype=np.int64).reshape(-1, 3)
     first, n = rows[:, 0], rows[:, 2]
     k = -(-n // per)
@@ -1421,11 +1422,12 @@ class HipOps:
             items, n_items = plan[0].reshape(-1), plan[1]
             if items.numel() < 2 * n_items or items.dtype != torch.int32 or not items.is_contiguous():
                 raise KernelError(f"attention: a list of {items.numel()} integers for {n_items} items")
-        # enough waves to fill the chip: a request's keys are cut where its items alone would leave most units idle
+        # Portions: the four-wave kernel, every item's keys whole. Single rows: a wave per row and 16 heads, with
+        # enough waves to fill the chip: a request's keys are cut where its rows alone would leave most units idle
         waves = n_items * -(-n_heads // 16)
         steps = -(-batch.max_kv_len // 32)
         most = max(1, (self._workspace.numel() // (n * n_heads * (value_dim + 2))))
-        n_splits = int(max(1, min(-(-2 * self.units // waves), steps // 4, 64, most)))
+        n_splits = 0 if items is not None else int(max(1, min(-(-2 * self.units // waves), steps // 4, 64, most)))
         part_o = part_ml = None
         if n_splits > 1:
             part_o = self._workspace
