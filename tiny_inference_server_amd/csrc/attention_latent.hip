@@ -198,23 +198,43 @@ __global__ __launch_bounds__(256) void latent_tile_kernel(
   constexpr int KP = KD / 8;                                    // 16-byte pieces of a key
   constexpr int VP = VD * PAGE / 8;                             // ... of a page's values
 
-  for (int s = 0; s < n_steps; ++s) {
+  // A thread's pieces of a step's keys and values, fetched into registers a step ahead (all loads issued together,
+  // in flight while the step before is computed) and put into LDS between two barriers.
+  constexpr int KN = (32 * KP + 255) / 256, VN = (2 * VP + 255) / 256;
+  bf16x8 kreg[KN], vreg[VN];
+  auto fetch = [&](int s) {
     const int kb = s * 32;
     const bool ok1 = kb + 16 <= p_last;
     const bf16* pg0 = plane + (long)bt[kb >> 4] * page_stride;
     const bf16* pg1 = plane + (long)(ok1 ? bt[(kb >> 4) + 1] : bt[kb >> 4]) * page_stride;
-    __syncthreads();                                            // everyone has read the step before
-    for (int i = tid; i < 32 * KP; i += 256) {
-      const int key = i / KP, piece = i % KP;
-      const bf16* src = (key < 16 ? pg0 : pg1) + (long)(key & 15) * KD + piece * 8;
-      *reinterpret_cast<bf16x8*>(k_lds + key * TK_STRIDE + piece * 8) = *reinterpret_cast<const bf16x8*>(src);
+#pragma unroll
+    for (int j = 0; j < KN; ++j) {
+      const int i = tid + j * 256, key = i / KP, piece = i % KP;
+      if (i < 32 * KP) kreg[j] = *reinterpret_cast<const bf16x8*>((key < 16 ? pg0 : pg1) + (long)(key & 15) * KD + piece * 8);
     }
-    for (int i = tid; i < 2 * VP; i += 256) {
-      const int pgi = i / VP, piece = i % VP;
-      const bf16* src = (pgi ? pg1 : pg0) + (long)PAGE * KD + piece * 8;
-      *reinterpret_cast<bf16x8*>(v_lds + pgi * VD * PAGE + piece * 8) = *reinterpret_cast<const bf16x8*>(src);
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      const int i = tid + j * 256, pgi = i / VP, piece = i % VP;
+      if (i < 2 * VP) vreg[j] = *reinterpret_cast<const bf16x8*>((pgi ? pg1 : pg0) + (long)PAGE * KD + piece * 8);
+    }
+  };
+  fetch(0);
+  for (int s = 0; s < n_steps; ++s) {
+    const int kb = s * 32;
+    const bool ok1 = kb + 16 <= p_last;
+    __syncthreads();                                            // everyone has read the step before
+#pragma unroll
+    for (int j = 0; j < KN; ++j) {
+      const int i = tid + j * 256, key = i / KP, piece = i % KP;
+      if (i < 32 * KP) *reinterpret_cast<bf16x8*>(k_lds + key * TK_STRIDE + piece * 8) = kreg[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VN; ++j) {
+      const int i = tid + j * 256;
+      if (i < 2 * VP) *reinterpret_cast<bf16x8*>(v_lds + i * 8) = vreg[j];
     }
     __syncthreads();
+    if (s + 1 < n_steps) fetch(s + 1);
     f32x4 st0 = {0.f, 0.f, 0.f, 0.f}, st1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int dc = 0; dc < DC; ++dc) {
