@@ -117,7 +117,10 @@ class Model:
             for i, call in enumerate(st.calls):
                 keys = self.call_keys[j][i]
                 # the rows going into a layer are replaced by its result: the layer may overwrite them
-                ctx = CallContext(batch=b, writes_cache=call.writes_cache, residual_is_spent=True)
+                after = st.calls[i + 1].layer if i + 1 < len(st.calls) else None
+                ctx = CallContext(batch=b, writes_cache=call.writes_cache, residual_is_spent=True,
+                                  next_norm=getattr(self.layers[after], "first_norm", None) if after is not None
+                                  else self.out_norms[j])
                 if len(keys) == 1:
                     self._bind(ctx, next(iter(keys.values())), cache)
                 elif keys:

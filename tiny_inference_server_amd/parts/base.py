@@ -67,6 +67,9 @@ class CallContext:
     state: Any = None                # [max requests, *shape] for state needs
     writes_cache: bool = True
     residual_is_spent: bool = False  # the caller will not read the residual it passes again: it may be overwritten
+    next_norm: Any = None            # the norm part that reads this call's result next (the following block's first
+                                     # norm, as it says in `first_norm`, or the stage's closing norm), if known: a block
+                                     # may fuse it into its last kernel
     bindings: Optional[Dict[str, "CallContext"]] = None     # per mixer part of the block
 
     def of(self, part_name: str) -> "CallContext":

@@ -35,6 +35,8 @@ class LayerNorm:
         return "layer", self.gain, self.bias, self.eps
 
     def __call__(self, x):
+        if isinstance(x, Stream32) and x.normed_by is self:
+            return x.rows               # the block before has applied this norm in its last kernel
         return self.ops.layernorm32(x.full if isinstance(x, Stream32) else x, self.gain, self.bias, self.eps)
 
 
@@ -89,6 +91,7 @@ class PreNormStream32(Arrangement):
         self.norm_a, self.mixer = self.parts["mixer_norm"], self.parts["mixer"]
         self.ffn, self.norm_f = self.parts.get("feed_forward"), self.parts.get("feed_forward_norm")
         self.side = self.parts.get("token_input")
+        self.first_norm = self.norm_a       # what reads this block's input first: the block before may apply it
         if (self.ffn is None) != (self.norm_f is None):
             raise ValueError("a prenorm_stream32 block has a feed-forward and its norm, or neither")
 
@@ -102,13 +105,16 @@ class PreNormStream32(Arrangement):
 
     def forward(self, x, ctx):
         x32 = x.full
-        y = self.mixer.forward32(self.norm_a(x32), ctx.of("mixer"))
-        rows = None
+        y = self.mixer.forward32(self.norm_a(x), ctx.of("mixer"))
         if self.ffn is not None:
             x32, _, h = self._sum(x32, y, norm=self.norm_f)
             y = self.ffn.forward32(h)
-        x32, rows, _ = self._sum(x32, y, copy=self.side is not None)
-        if self.side is not None:
+        # the block's last sum also applies the norm that reads its result next, where that norm can be fused
+        after = ctx.next_norm if hasattr(ctx.next_norm, "fused") else None
+        if self.side is None:
+            x32, _, normed = self._sum(x32, y, norm=after)
+        else:
+            x32, rows, _ = self._sum(x32, y, copy=True)
             y, y_rms = self.side.forward(rows, ctx.batch.tokens)
-            x32, rows, _ = self._sum(x32, y, y_rms=y_rms)
-        return Stream32(x32, rows)
+            x32, _, normed = self._sum(x32, y, y_rms=y_rms, norm=after)
+        return Stream32(x32, normed, normed_by=after)

@@ -12,10 +12,13 @@ from .base import ARRANGEMENTS, FEED_FORWARDS, GATES, NORMS, STAGE_INPUTS, Arran
 
 
 class Stream32:
-    __slots__ = ("full", "rows")
+    __slots__ = ("full", "rows", "normed_by")
 
-    def __init__(self, full, rows):
+    def __init__(self, full, rows, normed_by=None):
         self.full, self.rows = full, rows        # [rows, width] float32; the same in the compute type
+        # a block that was told which norm reads its result next (CallContext.next_norm) may apply it in its last
+        # kernel: `rows` then holds that norm's result, and the norm part named here hands it on instead of running
+        self.normed_by = normed_by
 
 
 @STAGE_INPUTS.register("scaled_token_embedding")
