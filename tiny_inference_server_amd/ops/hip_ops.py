@@ -1427,7 +1427,9 @@ class HipOps:
         waves = n_items * -(-n_heads // 16)
         steps = -(-batch.max_kv_len // 32)
         most = max(1, (self._workspace.numel() // (n * n_heads * (value_dim + 2))))
-        n_splits = 0 if items is not None else int(max(1, min(-(-2 * self.units // waves), steps // 4, 64, most)))
+        # (a wave's step is two or three dependent trips to memory and little else, so many short chains beat few long
+        # ones: four waves a compute unit, down to one step each)
+        n_splits = 0 if items is not None else int(max(1, min(-(-4 * self.units // waves), steps, 64, most)))
         part_o = part_ml = None
         if n_splits > 1:
             part_o = self._workspace
