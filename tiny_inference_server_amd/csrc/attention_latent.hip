@@ -302,23 +302,47 @@ __global__ __launch_bounds__(256) void latent_tile_kernel(
 // out[row, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s over a (row, head)'s splits, in a fixed order
 __global__ __launch_bounds__(256) void latent_merge_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
                                                            bf16* __restrict__ out, long ldo, int H, int n_splits) {
+  __shared__ float w[256];                 // the weights of up to 256 splits at a time
+  __shared__ float red[16];
   const long row = blockIdx.x;
-  const int head = blockIdx.y;
+  const int head = blockIdx.y, t = threadIdx.x;
   const long base = (row * H + head) * n_splits;
   float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[base + s].x);
+  for (int s = t; s < n_splits; s += 256) M = fmaxf(M, part_ml[base + s].x);
+  M = block_max(M, red);
   float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float2 ml = part_ml[base + s];
-    if (ml.x != -INFINITY) L += exp2f(ml.x - M) * ml.y;
-  }
-  for (int c = threadIdx.x; c < VD; c += 256) {
-    float acc = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float mx = part_ml[base + s].x;
-      if (mx != -INFINITY) acc += exp2f(mx - M) * part_o[(base + s) * VD + c];
+  float acc[(VD + 255) / 256];
+#pragma unroll
+  for (int j = 0; j < (VD + 255) / 256; ++j) acc[j] = 0.f;
+  for (int s0 = 0; s0 < n_splits; s0 += 256) {
+    const int cnt = min(256, n_splits - s0);
+    float mine = 0.f, share = 0.f;
+    if (t < cnt) {
+      const float2 ml = part_ml[base + s0 + t];
+      if (ml.x != -INFINITY) {             // else: a split that held no key of this row (its partial output is zero)
+        mine = exp2f(ml.x - M);
+        share = mine * ml.y;
+      }
     }
-    out[row * ldo + (long)head * VD + c] = static_cast<__bf16>(acc / L);
+    __syncthreads();
+    w[t] = mine;
+    L += block_sum(share, red);            // its barriers also publish w[]
+    // (a split's partial outputs are independent loads: several are in flight at a time)
+#pragma unroll
+    for (int j = 0; j < (VD + 255) / 256; ++j) {
+      const int c = j * 256 + t;
+      if (c >= VD) continue;
+      const float* src = part_o + (base + s0) * VD + c;
+      float a = 0.f;
+#pragma unroll 8
+      for (int s = 0; s < cnt; ++s) a += w[s] * src[(long)s * VD];
+      acc[j] += a;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < (VD + 255) / 256; ++j) {
+    const int c = j * 256 + t;
+    if (c < VD) out[row * ldo + (long)head * VD + c] = static_cast<__bf16>(acc[j] / L);
   }
 }
 
