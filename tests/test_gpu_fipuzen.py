@@ -55,7 +55,7 @@ def close(a, b, dtype, what, tol=None):
 
 # ---- kernels ---------------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("D", [44, 300, 1500])
+@pytest.mark.parametrize("D", [44, 300, 1500, 4200])      # (a row in 4 or 16 registers a thread, or in memory)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_sums_and_norms_of_the_stream(dtype, D):
     ops, ref = hip_ops(dtype), TorchOps("cpu", DT[dtype])

@@ -162,45 +162,84 @@ __global__ __launch_bounds__(S32_THREADS) void layernorm32_kernel(const float* _
 //   v = x + y / sqrt(mean(y^2) + y_eps) * y_gain   (an RMS norm on the branch before the sum)
 // v goes to out32 (which may be x itself); `copy` (nullable) gets v in the compute type; `normed` (nullable) gets the
 // norm of v in the compute type: kind 1 layer norm (gain, bias), kind 2 RMS norm (gain), eps under the root in both.
-template <typename T>
+// PER: values a thread keeps in registers (width <= 256 * PER), so that the row is read once and the sums follow one
+// another without a trip to memory between them; 0: any width, through out32.
+template <typename T, int PER>
 __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
     const float* __restrict__ x, const float* __restrict__ y, long ldy, const float* __restrict__ y_gain, float y_eps,
     float* __restrict__ out32, T* __restrict__ copy, long ldc, int norm_kind, const float* __restrict__ gain,
     const float* __restrict__ bias, float eps, T* __restrict__ normed, long ldn, int D) {
   __shared__ float red[16];
   const long r = blockIdx.x;
+  constexpr int P = PER > 0 ? PER : 1;
+  float xv[P], yv[P];
+  if (PER > 0) {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int c = threadIdx.x + k * S32_THREADS;
+      xv[k] = c < D ? x[r * D + c] : 0.f;
+      yv[k] = (y && c < D) ? y[r * ldy + c] : 0.f;
+    }
+  }
   float y_inv = 1.f;
   if (y && y_gain) {
     float ss = 0.f;
-    for (int c = threadIdx.x; c < D; c += S32_THREADS) {
-      const float v = y[r * ldy + c];
-      ss += v * v;
+    if (PER > 0) {
+#pragma unroll
+      for (int k = 0; k < PER; ++k) ss += yv[k] * yv[k];
+    } else {
+      for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+        const float v = y[r * ldy + c];
+        ss += v * v;
+      }
     }
     y_inv = 1.f / sqrtf(block_sum(ss, red) / (float)D + y_eps);
   }
   float s = 0.f;
-  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
-    float v = x[r * D + c];
-    if (y) v += y_gain ? y[r * ldy + c] * y_inv * y_gain[c] : y[r * ldy + c];
-    out32[r * D + c] = v;          // (each thread reads back only what it wrote itself)
-    if (copy) copy[r * ldc + c] = from_f<T>(v);
-    s += norm_kind == 2 ? v * v : v;
+  if (PER > 0) {
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int c = threadIdx.x + k * S32_THREADS;
+      if (c >= D) continue;
+      float v = xv[k];
+      if (y) v += y_gain ? yv[k] * y_inv * y_gain[c] : yv[k];
+      xv[k] = v;
+      out32[r * D + c] = v;
+      if (copy) copy[r * ldc + c] = from_f<T>(v);
+      s += norm_kind == 2 ? v * v : v;
+    }
+  } else {
+    for (int c = threadIdx.x; c < D; c += S32_THREADS) {
+      float v = x[r * D + c];
+      if (y) v += y_gain ? y[r * ldy + c] * y_inv * y_gain[c] : y[r * ldy + c];
+      out32[r * D + c] = v;          // (each thread reads back only what it wrote itself)
+      if (copy) copy[r * ldc + c] = from_f<T>(v);
+      s += norm_kind == 2 ? v * v : v;
+    }
   }
   if (!normed || norm_kind == 0) return;
+  // every value of the row that this thread holds, from its registers or from what it wrote to out32
+  auto each = [&](auto fn) {
+    if (PER > 0) {
+#pragma unroll
+      for (int k = 0; k < P; ++k) {
+        const int c = threadIdx.x + k * S32_THREADS;
+        if (c < D) fn(xv[k], c);
+      }
+    } else {
+      for (int c = threadIdx.x; c < D; c += S32_THREADS) fn(out32[r * D + c], c);
+    }
+  };
   if (norm_kind == 2) {
     const float inv = 1.f / sqrtf(block_sum(s, red) / (float)D + eps);
-    for (int c = threadIdx.x; c < D; c += S32_THREADS) normed[r * ldn + c] = from_f<T>(out32[r * D + c] * inv * gain[c]);
+    each([&](float v, int c) { normed[r * ldn + c] = from_f<T>(v * inv * gain[c]); });
     return;
   }
   const float mean = block_sum(s, red) / (float)D;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < D; c += S32_THREADS) {
-    const float d = out32[r * D + c] - mean;
-    ss += d * d;
-  }
+  each([&](float v, int c) { ss += (v - mean) * (v - mean); });
   const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)D + eps);
-  for (int c = threadIdx.x; c < D; c += S32_THREADS)
-    normed[r * ldn + c] = from_f<T>((out32[r * D + c] - mean) * inv * gain[c] + (bias ? bias[c] : 0.f));
+  each([&](float v, int c) { normed[r * ldn + c] = from_f<T>((v - mean) * inv * gain[c] + (bias ? bias[c] : 0.f)); });
 }
 
 __device__ __forceinline__ float gelu_tanh_f(float z) {
@@ -322,10 +361,16 @@ TIS_EXPORT int tis_residual_norm(int dtype, const float* x, const float* y, long
   if (rows < 0 || D < 1 || !x || !out32) return tis_fail("residual_norm: bad arguments rows=%d width=%d", rows, D);
   if (norm_kind < 0 || norm_kind > 2 || (norm_kind && (!gain || !normed)))
     return tis_fail("residual_norm: norm kind %d needs a gain and an output", norm_kind);
-  S32_DISPATCH((residual_norm_kernel<float><<<rows, S32_THREADS, 0, stream>>>(x, y, ldy, y_gain, y_eps, out32, (float*)copy, ldc,
-                                                                             norm_kind, gain, bias, eps, (float*)normed, ldn, D)),
-               (residual_norm_kernel<bf16><<<rows, S32_THREADS, 0, stream>>>(x, y, ldy, y_gain, y_eps, out32, (bf16*)copy, ldc,
-                                                                            norm_kind, gain, bias, eps, (bf16*)normed, ldn, D)))
+#define S32_RESIDUAL(T, PER)                                                                                              \
+  residual_norm_kernel<T, PER><<<rows, S32_THREADS, 0, stream>>>(x, y, ldy, y_gain, y_eps, out32, (T*)copy, ldc, norm_kind, \
+                                                                 gain, bias, eps, (T*)normed, ldn, D)
+#define S32_RESIDUAL_BY_WIDTH(T)                         \
+  if (D <= 4 * S32_THREADS) { S32_RESIDUAL(T, 4); }      \
+  else if (D <= 16 * S32_THREADS) { S32_RESIDUAL(T, 16); } \
+  else { S32_RESIDUAL(T, 0); }
+  S32_DISPATCH(S32_RESIDUAL_BY_WIDTH(float), S32_RESIDUAL_BY_WIDTH(bf16))
+#undef S32_RESIDUAL_BY_WIDTH
+#undef S32_RESIDUAL
   return tis_launch_status("residual_norm");
 }
 
