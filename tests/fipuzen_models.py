@@ -73,7 +73,10 @@ def _configs():
     D = config(48, 77, [moe(lightning(2, 12, 8, (0.9, 0.6)), 32, 2, 0, 1, 1.0), moe(lightning(4, 4, 16, (1.0, 0.5, 0.99, 0.7)), None, 0, 0, 0, 0)],
                side=5)
     E = config(56, 150, [moe(attention(3, 3, 20, 36, 0.22), 48, 7, 0, 3, 1.3), moe(attention(2, 1, 40, 16, 0.16, 0.5, 3), None, 0, 0, 0, 0)])
-    return {"A": A, "B": B, "C": C, "D": D, "E": E}
+    # attention over a latent first (sizes that the matrix-core kernel takes), then grouped-query attention
+    F = config(96, 180, [moe(latent(4, 32, 16, 32, 64, 0.14, base=5e4), 48, 4, 1, 2, 1.5), moe(attention(2, 1, 16, 16, 0.25, 0.3, 64), None, 0, 0, 0, 0)],
+               side=6)
+    return {"A": A, "B": B, "C": C, "D": D, "E": E, "F": F}
 
 
 CONFIGS = _configs()
@@ -228,7 +231,19 @@ def sharpen(cfg, tensors, needle: int, probe: int, strength: float = 6.0):
     elif e["type"] == "lightning":
         t["l0.mix.q"] = looking(t["l0.mix.k"])
     else:
-        raise ValueError("the needle construction is for attention and lightning first layers")
+        # a head's unrotated query becomes its own unrotated key of the needle: Wuk[h] applied to the needle's latent
+        # (the gain times the latent's rows, behind the map from the probe to the needle; the norm's factor is a
+        # number per position and goes into the strength)
+        H, D, R, C = m["heads"], m["dim"], m["rot_dim"], m["kv_rank"]
+        rows = looking(t["l0.mix.dkv.norm"][:, None] * t["l0.mix.dkv"][:C])            # [C, width]
+        uk = t["l0.mix.uk"].view(H, D, C)
+        q = t["l0.mix.q"].view(H, D + R, -1).clone()
+        down = t["l0.mix.dkv"][:C] @ hn
+        c_n = down / torch.sqrt((down * down).mean() + eps) * t["l0.mix.dkv.norm"]
+        hit = torch.stack([(uk[h] @ rows @ hp) @ (uk[h] @ c_n) for h in range(H)]).mean()
+        for h in range(H):
+            q[h, :D] = uk[h] @ rows * (strength / m["scale"] / float(hit))
+        t["l0.mix.q"] = q.reshape(H * (D + R), -1)
     return {n: v.to(tensors[n].dtype) for n, v in t.items()}
 
 

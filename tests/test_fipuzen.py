@@ -211,7 +211,7 @@ def needle_case(name, distance, at, length=None, seed=60):
     return cfg, w, w64, ids, moved
 
 
-@pytest.mark.parametrize("name,distance", [("A", 1), ("A", 300), ("E", 200), ("D", 150)])
+@pytest.mark.parametrize("name,distance", [("A", 1), ("A", 300), ("E", 200), ("D", 150), ("F", 1), ("F", 250)])
 def test_a_token_that_stands_out(name, distance):
     """The probe looks for a needle right before it or hundreds of tokens back (through attention's pages or a
     recurrent state), with the needle on both sides of a page's border; whole, decoded alone and in portions."""

@@ -225,7 +225,7 @@ def test_routing_in_bfloat16():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,distance", [("A", 1), ("A", 300), ("E", 200), ("D", 150)])
+@pytest.mark.parametrize("name,distance", [("A", 1), ("A", 300), ("E", 200), ("D", 150), ("F", 1), ("F", 250)])
 def test_a_token_that_stands_out(name, distance, dtype):
     """A probe token that looks for a needle right before it or hundreds of tokens back, through attention's pages or a
     recurrent state, with the needle on both sides of a page's border: whole, decoded alone, in portions."""
