@@ -50,6 +50,19 @@ def test_spec_names_every_tensor(tmp_path):
             assert ("token_input" in layer.parts) == ("token_side" in cfg)
 
 
+def test_a_side_table_wider_than_the_layers_need(tmp_path):
+    """Layer i reads the columns [i * dim, (i + 1) * dim) of the side table; the table's width comes from the file."""
+    cfg, w, _ = model("D")
+    w = dict(w)
+    w["side.embed"] = torch.cat((w["side.embed"], torch.randn(cfg["vocab"], 3).to(w["side.embed"].dtype)), dim=1)
+    folder = ZM.write_folder(str(tmp_path / "wide"), cfg, w)
+    assert load_config(folder).side_width == w["side.embed"].shape[1]
+    eng = Engine(folder, dtype="float32", max_tokens=64, max_requests=2, page_size=8, ops=TorchOps())
+    ids = H.random_ids(cfg["vocab"], 20, 3)
+    got = ZM.run_trace(eng, H.whole_trace({"a": ids}))
+    assert ZM.worst_error("Dwide", cfg, ZM.as_f64(w), {"a": ids}, got)[0] <= TOL32
+
+
 def test_configuration_errors_name_the_key():
     good = ZM.CONFIGS["A"]
     for path, value, word in [(("layers", 0, "type"), "conv", "type"), (("layers", 0, "mixer", "kv_heads"), 3, "kv_heads"),

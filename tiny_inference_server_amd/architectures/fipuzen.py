@@ -71,7 +71,7 @@ def _block(cfg, entry, i):
         parts["feed_forward_norm"] = _norm(cfg, pre + "norm2")
         parts["feed_forward"] = _experts(cfg, entry["mlp"], pre + "mlp.")
     if cfg.side_dim:
-        params = {"width": cfg.width, "dim": cfg.side_dim, "vocab": cfg.vocab, "table_width": cfg.side_dim * len(cfg.layers),
+        params = {"width": cfg.width, "dim": cfg.side_dim, "vocab": cfg.vocab, "table_width": cfg.side_width,
                   "offset": i * cfg.side_dim, "eps": cfg.norm_eps, "act": "gelu_tanh"}
         parts["token_input"] = PartSpec("token_input", "gated_token_table", params,
                                         {"table": "side.embed", "gate": pre + "side.gate", "proj": pre + "side.proj",

@@ -70,6 +70,7 @@ class FipuzenConfig:
     layers: Tuple[Dict[str, Any], ...]
     architecture: str = "Fipuzen"
     extra: Dict[str, Any] = field(default_factory=dict, compare=False)
+    side_table_width: int = 0          # columns of the side table; 0: side_dim * layers (a file's table may be wider)
 
     def __post_init__(self):
         _need(self.vocab >= 1 and self.width >= 1, f"vocab {self.vocab} and width {self.width} must be at least 1")
@@ -90,6 +91,19 @@ class FipuzenConfig:
                    layers=tuple(copy.deepcopy(dict(e)) if isinstance(e, Mapping) else e for e in raw["layers"]),
                    architecture=str(raw.get("architecture", "Fipuzen")),
                    extra={k: v for k, v in raw.items() if k not in used})
+
+    @property
+    def side_width(self) -> int:
+        return self.side_table_width or self.side_dim * len(self.layers)
+
+    def with_tensor_shapes(self, shapes: Mapping[str, Tuple[int, ...]]) -> "FipuzenConfig":
+        """The same configuration with the side table's width as the weight file has it (layer i reads the columns
+        [i * dim, (i + 1) * dim), whatever lies beyond the last layer's)."""
+        shape = shapes.get("side.embed")
+        if not self.side_dim or shape is None or len(shape) != 2 or shape[1] < self.side_dim * len(self.layers):
+            return self
+        return FipuzenConfig(self.vocab, self.width, self.norm_eps, self.side_dim, self.layers, self.architecture,
+                             dict(self.extra), int(shape[1]))
 
     def to_dict(self) -> Dict[str, Any]:
         out = {"architecture": self.architecture, "vocab": self.vocab, "width": self.width, "norm": {"eps": self.norm_eps},
