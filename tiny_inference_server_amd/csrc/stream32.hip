@@ -172,13 +172,18 @@ __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
   __shared__ float red[16];
   const long r = blockIdx.x;
   constexpr int P = PER > 0 ? PER : 1;
-  float xv[P], yv[P];
+  // (everything the row's columns need is asked for at once: the gains and the bias too, which are only used after
+  // the sums, so that no trip to memory stands between two of them)
+  float xv[P], yv[P], ygv[P], gv[P], bv[P];
   if (PER > 0) {
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
       const int c = threadIdx.x + k * S32_THREADS;
       xv[k] = c < D ? x[r * D + c] : 0.f;
       yv[k] = (y && c < D) ? y[r * ldy + c] : 0.f;
+      ygv[k] = (y && y_gain && c < D) ? y_gain[c] : 1.f;
+      gv[k] = (norm_kind && c < D) ? gain[c] : 0.f;
+      bv[k] = (norm_kind == 1 && bias && c < D) ? bias[c] : 0.f;
     }
   }
   float y_inv = 1.f;
@@ -202,7 +207,7 @@ __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
       const int c = threadIdx.x + k * S32_THREADS;
       if (c >= D) continue;
       float v = xv[k];
-      if (y) v += y_gain ? yv[k] * y_inv * y_gain[c] : yv[k];
+      if (y) v += y_gain ? yv[k] * y_inv * ygv[k] : yv[k];
       xv[k] = v;
       out32[r * D + c] = v;
       if (copy) copy[r * ldc + c] = from_f<T>(v);
@@ -218,28 +223,28 @@ __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
     }
   }
   if (!normed || norm_kind == 0) return;
-  // every value of the row that this thread holds, from its registers or from what it wrote to out32
+  // every value of the row that this thread holds (with its gain and bias), from its registers or from memory
   auto each = [&](auto fn) {
     if (PER > 0) {
 #pragma unroll
       for (int k = 0; k < P; ++k) {
         const int c = threadIdx.x + k * S32_THREADS;
-        if (c < D) fn(xv[k], c);
+        if (c < D) fn(xv[k], c, gv[k], bv[k]);
       }
     } else {
-      for (int c = threadIdx.x; c < D; c += S32_THREADS) fn(out32[r * D + c], c);
+      for (int c = threadIdx.x; c < D; c += S32_THREADS) fn(out32[r * D + c], c, gain[c], (norm_kind == 1 && bias) ? bias[c] : 0.f);
     }
   };
   if (norm_kind == 2) {
     const float inv = 1.f / sqrtf(block_sum(s, red) / (float)D + eps);
-    each([&](float v, int c) { normed[r * ldn + c] = from_f<T>(v * inv * gain[c]); });
+    each([&](float v, int c, float g, float) { normed[r * ldn + c] = from_f<T>(v * inv * g); });
     return;
   }
   const float mean = block_sum(s, red) / (float)D;
   float ss = 0.f;
-  each([&](float v, int c) { ss += (v - mean) * (v - mean); });
+  each([&](float v, int, float, float) { ss += (v - mean) * (v - mean); });
   const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)D + eps);
-  each([&](float v, int c) { normed[r * ldn + c] = from_f<T>((v - mean) * inv * gain[c] + (bias ? bias[c] : 0.f)); });
+  each([&](float v, int c, float g, float b) { normed[r * ldn + c] = from_f<T>((v - mean) * inv * g + b); });
 }
 
 __device__ __forceinline__ float gelu_tanh_f(float z) {
