@@ -183,6 +183,15 @@ def test_router_and_experts(dtype, n, W, F, E, I, top):
     got = ops.routed_experts(x.cuda(), ids, wts, up.cuda() if E else None, down.cuda() if E else None)
     want = ref.routed_experts(x, ids.cpu(), wts.cpu(), up, down)
     close(got, want, dtype, "experts")
+    # the same sum taken inside the residual sum's kernel, with the norm that follows
+    x32, gain = torch.randn(n, W, generator=g), 1 + 0.1 * torch.randn(W, generator=g)
+    a = ops.residual_norm(x32.cuda(), ops.routed_experts(x.cuda(), ids, wts, up.cuda() if E else None, down.cuda() if E else None,
+                                                         combine=False), copy=True, norm=("layer", gain.cuda(), None, 1e-5))
+    b = ref.residual_norm(x32.clone(), ref.routed_experts(x, ids.cpu(), wts.cpu(), up, down, combine=False), copy=True,
+                          norm=("layer", gain, None, 1e-5))
+    for u, v, what in zip(a, b, ("sum with experts", "its copy", "its norm")):
+        close(u, v, dtype, what)
+    close(a[0], x32 + want.float(), dtype, "sum with experts against the separate sum")
     # a tie goes to the lower index
     tie = torch.zeros(2, 5).cuda()
     ids, _ = ops.route_topk(tie, None, 1.0, 2)

@@ -299,6 +299,11 @@ class TorchOps:
         return (y + bias if bias is not None else y).to(self.dtype)
 
     def residual_norm(self, x32, y=None, y_rms=None, copy=False, norm=None):
+        if isinstance(y, tuple) and hasattr(y, "n_experts"):           # the experts' results, not summed yet
+            n, top = y.ids.shape
+            parts = y.results.view(n, top, -1) if y.results is not None else torch.zeros(n, top, x32.shape[1])
+            own = (y.ids >= y.n_experts)[:, :, None]
+            y = (y.weights[:, :, None] * torch.where(own, y.rows.float()[:, None, :], parts)).sum(1)
         if y is not None:
             y = y.float()[:, :x32.shape[1]]
             if y_rms is not None:
@@ -338,20 +343,22 @@ class TorchOps:
         ids = torch.topk(choice, top, dim=-1).indices
         return ids.to(torch.int32), torch.gather(s, 1, ids) * scale
 
-    def routed_experts(self, x, ids, weights, w_up, w_down, act="gelu_erf"):
+    def routed_experts(self, x, ids, weights, w_up, w_down, act="gelu_erf", combine=True):
+        from tiny_inference_server_amd.ops.hip_ops import ChosenExperts
         E = w_up.shape[0] if w_up is not None else 0
         xf = x.float()
-        out = torch.zeros_like(xf)
-        for r in range(x.shape[0]):
-            for k in range(ids.shape[1]):
+        n, top = ids.shape
+        parts = torch.zeros(n * top, x.shape[1])
+        for r in range(n):
+            for k in range(top):
                 e = int(ids[r, k])
-                if e >= E:
-                    y = xf[r]
-                else:
+                if e < E:
                     hid = torch.nn.functional.gelu(w_up[e].float() @ xf[r]).to(self.dtype).float()
-                    y = w_down[e].float() @ hid
-                out[r] += weights[r, k] * y
-        return out
+                    parts[r * top + k] = w_down[e].float() @ hid
+        if not combine:
+            return ChosenExperts(parts if E else None, ids, weights, E, x)
+        own = (ids >= E)[:, :, None]
+        return (weights[:, :, None] * torch.where(own, xf[:, None, :], parts.view(n, top, -1))).sum(1)
 
     @staticmethod
     def state_scan_floats(kind, n_heads, dim, vdim):

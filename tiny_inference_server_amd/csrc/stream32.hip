@@ -162,16 +162,38 @@ __global__ __launch_bounds__(S32_THREADS) void layernorm32_kernel(const float* _
 //   v = x + y / sqrt(mean(y^2) + y_eps) * y_gain   (an RMS norm on the branch before the sum)
 // v goes to out32 (which may be x itself); `copy` (nullable) gets v in the compute type; `normed` (nullable) gets the
 // norm of v in the compute type: kind 1 layer norm (gain, bias), kind 2 RMS norm (gain), eps under the root in both.
+// Where the branch is a routed feed-forward's result that has not been summed yet: y then holds a line per (row, choice),
+// and the branch's value at row r is sum_k weights[r][k] * (y[r * top + k] if ids[r][k] < n_experts else rows[r]): an
+// id from n_experts on is an identity expert, whose result is the row it was given. ids null: y is the branch itself.
+struct ChosenSum {
+  const int* ids;
+  const float* weights;
+  int top, n_experts;
+  const void* rows;      // [rows][ldr] in the compute type: what the feed-forward read
+  long ldr;
+};
+
 // PER: values a thread keeps in registers (width <= 256 * PER), so that the row is read once and the sums follow one
 // another without a trip to memory between them; 0: any width, through out32.
 template <typename T, int PER>
 __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
-    const float* __restrict__ x, const float* __restrict__ y, long ldy, const float* __restrict__ y_gain, float y_eps,
+    const float* __restrict__ x, const float* __restrict__ y_in, long ldy, const float* __restrict__ y_gain, float y_eps,
     float* __restrict__ out32, T* __restrict__ copy, long ldc, int norm_kind, const float* __restrict__ gain,
-    const float* __restrict__ bias, float eps, T* __restrict__ normed, long ldn, int D) {
+    const float* __restrict__ bias, float eps, T* __restrict__ normed, long ldn, int D, ChosenSum cs) {
   __shared__ float red[16];
   const long r = blockIdx.x;
   constexpr int P = PER > 0 ? PER : 1;
+  const bool y = y_in != nullptr || cs.ids != nullptr;        // whether there is a branch at all
+  auto y_at = [&](int c) {
+    if (!cs.ids) return y_in[r * ldy + c];
+    float v = 0.f;
+    for (int k = 0; k < cs.top; ++k) {
+      const float w = cs.weights[r * cs.top + k];
+      v += w * (cs.ids[r * cs.top + k] < cs.n_experts ? y_in[(r * cs.top + k) * ldy + c]
+                                                        : to_f(static_cast<const T*>(cs.rows)[r * cs.ldr + c]));
+    }
+    return v;
+  };
   // (everything the row's columns need is asked for at once: the gains and the bias too, which are only used after
   // the sums, so that no trip to memory stands between two of them)
   float xv[P], yv[P], ygv[P], gv[P], bv[P];
@@ -180,7 +202,7 @@ __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
     for (int k = 0; k < PER; ++k) {
       const int c = threadIdx.x + k * S32_THREADS;
       xv[k] = c < D ? x[r * D + c] : 0.f;
-      yv[k] = (y && c < D) ? y[r * ldy + c] : 0.f;
+      yv[k] = (y && c < D) ? y_at(c) : 0.f;
       ygv[k] = (y && y_gain && c < D) ? y_gain[c] : 1.f;
       gv[k] = (norm_kind && c < D) ? gain[c] : 0.f;
       bv[k] = (norm_kind == 1 && bias && c < D) ? bias[c] : 0.f;
@@ -194,7 +216,7 @@ __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
       for (int k = 0; k < PER; ++k) ss += yv[k] * yv[k];
     } else {
       for (int c = threadIdx.x; c < D; c += S32_THREADS) {
-        const float v = y[r * ldy + c];
+        const float v = y_at(c);
         ss += v * v;
       }
     }
@@ -216,7 +238,7 @@ __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
   } else {
     for (int c = threadIdx.x; c < D; c += S32_THREADS) {
       float v = x[r * D + c];
-      if (y) v += y_gain ? y[r * ldy + c] * y_inv * y_gain[c] : y[r * ldy + c];
+      if (y) v += y_gain ? y_at(c) * y_inv * y_gain[c] : y_at(c);
       out32[r * D + c] = v;          // (each thread reads back only what it wrote itself)
       if (copy) copy[r * ldc + c] = from_f<T>(v);
       s += norm_kind == 2 ? v * v : v;
@@ -361,14 +383,18 @@ TIS_EXPORT int tis_layernorm32(int dtype, const float* x, const float* gain, con
 
 TIS_EXPORT int tis_residual_norm(int dtype, const float* x, const float* y, long ldy, const float* y_gain, float y_eps,
                                  float* out32, void* copy, long ldc, int norm_kind, const float* gain, const float* bias,
-                                 float eps, void* normed, long ldn, int rows, int D, hipStream_t stream) {
+                                 float eps, void* normed, long ldn, int rows, int D, const int* ids, const float* weights,
+                                 int top, int n_experts, const void* chosen_rows, long ldr, hipStream_t stream) {
   if (rows == 0) return 0;
   if (rows < 0 || D < 1 || !x || !out32) return tis_fail("residual_norm: bad arguments rows=%d width=%d", rows, D);
+  if (ids && (!weights || top < 1 || n_experts < 0 || (n_experts > 0 && !y) || !chosen_rows))
+    return tis_fail("residual_norm: a sum over chosen experts needs ids, weights, the experts' results and the rows they read");
+  const ChosenSum cs{ids, weights, top, n_experts, chosen_rows, ldr};
   if (norm_kind < 0 || norm_kind > 2 || (norm_kind && (!gain || !normed)))
     return tis_fail("residual_norm: norm kind %d needs a gain and an output", norm_kind);
 #define S32_RESIDUAL(T, PER)                                                                                              \
   residual_norm_kernel<T, PER><<<rows, S32_THREADS, 0, stream>>>(x, y, ldy, y_gain, y_eps, out32, (T*)copy, ldc, norm_kind, \
-                                                                 gain, bias, eps, (T*)normed, ldn, D)
+                                                                 gain, bias, eps, (T*)normed, ldn, D, cs)
 #define S32_RESIDUAL_BY_WIDTH(T)                         \
   if (D <= 4 * S32_THREADS) { S32_RESIDUAL(T, 4); }      \
   else if (D <= 16 * S32_THREADS) { S32_RESIDUAL(T, 16); } \

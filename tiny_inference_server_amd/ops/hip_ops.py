@@ -110,7 +110,7 @@ _SIGNATURES["stream32"] = ("tis_stream32", {
     "tis_head_norm_gate": [_I, _P, _L, _P, _L, _P, _I, _I, _F, _P, _L, _I, _I, _I, _P],
     "tis_lowrank_decay": [_P, _L, _I, _P, _P, _F, _P, _I, _I, _P],
     "tis_layernorm32": [_I, _P, _P, _P, _F, _P, _L, _I, _I, _P],
-    "tis_residual_norm": [_I, _P, _P, _L, _P, _F, _P, _P, _L, _I, _P, _P, _F, _P, _L, _I, _I, _P],
+    "tis_residual_norm": [_I, _P, _P, _L, _P, _F, _P, _P, _L, _I, _P, _P, _F, _P, _L, _I, _I, _P, _P, _I, _I, _P, _L, _P],
     "tis_gate_table": [_I, _P, _L, _P, _L, _P, _I, _P, _L, _I, _I, _P],
     "tis_activate32": [_P, _L, _I, _I, _I, _P],
     "tis_head_gate": [_I, _P, _L, _P, _L, _I, _I, _I, _P],
@@ -416,6 +416,15 @@ def latent_items(seq_rows, n_heads: int, columns: int = 64):
     r = (np.arange(int(k.sum())) - np.repeat(np.cumsum(k) - k, k)) * per
     counts = np.minimum(per, np.repeat(n, k) - r)
     return np.stack((np.repeat(first, k) + r, counts), axis=1).astype(np.int32)
+
+
+class ChosenExperts(NamedTuple):
+    """A routed feed-forward's result before the sum over a row's choices."""
+    results: Optional[torch.Tensor]     # [rows * top, width] 32-bit, a line per (row, choice); None with no real expert
+    ids: torch.Tensor                   # [rows, top] int32
+    weights: torch.Tensor               # [rows, top] 32-bit
+    n_experts: int                      # ids from here on are identity experts
+    rows: torch.Tensor                  # [rows, width] in the compute type: what the feed-forward read
 
 
 class AttentionLaunch(NamedTuple):
@@ -1177,13 +1186,28 @@ class HipOps:
     def residual_norm(self, x32, y=None, y_rms=None, copy=False, norm=None):
         """x32 <- x32 + y, in place, with what usually follows: (x32, copy, normed).
 
+        y may also be a `ChosenExperts` (what routed_experts gives with combine=False): the weighted sum of a row's
+        chosen experts is then taken inside this kernel.
+
         y: [rows, width] 32-bit (a strided view is fine) or None; y_rms = (gain, eps): y is RMS-normed with that gain
         before it is added. copy: also return the new rows in the compute type. norm = (kind, gain, bias, eps) with kind
         "layer" (bias may be None) or "rms": also return the norm of the new rows in the compute type. In a 32-bit
         engine the copy is the stream itself."""
         n, D = x32.shape
         self._f32(x32, "residual_norm x", n * D)
-        if y is not None:
+        chosen = None
+        if isinstance(y, ChosenExperts):
+            chosen, y = y, y.results
+            top = chosen.ids.shape[1]
+            self._index(chosen.ids, "expert ids", n * top)
+            self._f32(chosen.weights, "expert weights", n * top)
+            _rows_view(self._check(chosen.rows, "experts' input rows"), "experts' input rows")
+            if tuple(chosen.rows.shape) != (n, D) or (y is not None and tuple(y.shape) != (n * top, D)):
+                raise KernelError(f"residual_norm: experts' results {None if y is None else tuple(y.shape)} and rows "
+                                  f"{tuple(chosen.rows.shape)} for {n} rows of {D} with {top} choices")
+            if y is not None:
+                self._f32_rows(y, "experts' results", n * top, D)
+        elif y is not None:
             self._f32_rows(y, "residual_norm y", n, D)
         elif y_rms is not None:
             raise KernelError("residual_norm: a norm on a branch that is not there")
@@ -1202,7 +1226,10 @@ class HipOps:
         self._lazy("stream32").tis_residual_norm(
             self.code, _ptr(x32), _ptr(y), y.stride(0) if y is not None else 0, _ptr(y_rms[0] if y_rms else None),
             float(y_rms[1]) if y_rms else 0.0, _ptr(x32), _ptr(cp), cp.stride(0) if cp is not None else 0, kind, _ptr(gain),
-            _ptr(bias), float(eps), _ptr(normed), normed.stride(0) if normed is not None else 0, n, D, self._stream())
+            _ptr(bias), float(eps), _ptr(normed), normed.stride(0) if normed is not None else 0, n, D,
+            _ptr(chosen.ids if chosen else None), _ptr(chosen.weights if chosen else None),
+            chosen.ids.shape[1] if chosen else 0, chosen.n_experts if chosen else 0,
+            _ptr(chosen.rows if chosen else None), chosen.rows.stride(0) if chosen else 0, self._stream())
         return x32, (x32 if copy and as_is else cp), normed
 
     _ACTS = {"gelu_tanh": 0, "silu": 1, "sigmoid": 2}
@@ -1281,10 +1308,11 @@ class HipOps:
                                              _ptr(weights), self._stream())
         return ids, weights
 
-    def routed_experts(self, x, ids, weights, w_up, w_down, act: str = "gelu_erf"):
+    def routed_experts(self, x, ids, weights, w_up, w_down, act: str = "gelu_erf", combine: bool = True):
         """sum_k weights[:, k] * expert(ids[:, k])(x) in 32-bit: expert e < len(w_up) is w_down[e] . act(w_up[e] . x),
         any id beyond is an identity expert whose result is x itself. x: [rows, width] in the compute type; w_up
-        [experts, hidden, width], w_down [experts, width, hidden]."""
+        [experts, hidden, width], w_down [experts, width, hidden]. combine=False: the experts' results line by
+        (row, choice), not summed yet, as a `ChosenExperts` that residual_norm takes in place of a branch."""
         _rows_view(self._check(x, "experts x"), "experts x")
         n, D = x.shape
         top = ids.shape[1]
@@ -1306,6 +1334,8 @@ class HipOps:
             self._grouped(x, x.stride(0), 0, top, w_up, hidden, hidden.stride(0), 0, lists, counts, n, n, act=1)
             y = torch.empty(n * top, D, dtype=torch.float32, device=self.device)
             self._grouped(hidden, hidden.stride(0), 0, 1, w_down, y, D, 0, lists, counts, n, n)
+        if not combine:
+            return ChosenExperts(y, ids, weights, E, x)
         out = torch.empty(n, D, dtype=torch.float32, device=self.device)
         lib.tis_experts_combine(self.code, _ptr(y), D, _ptr(x), x.stride(0), _ptr(ids), _ptr(weights), top, E, _ptr(out), D,
                                 n, D, self._stream())

@@ -76,11 +76,15 @@ class RoutedExperts:
             self.w_up = to_compute(ops, torch.stack([tensors.of(spec, f"up{e}") for e in range(self.E)]))
             self.w_down = to_compute(ops, torch.stack([tensors.of(spec, f"down{e}") for e in range(self.E)]))
 
-    def forward32(self, x):
+    def forward32(self, x, combine=True):
+        """combine=False: the experts' results before the sum over a row's choices, for a residual sum that takes it
+        (what `ops.routed_experts(..., combine=False)` gives)."""
         ops = self.ops
         z = ops.linear(x, self.w_router, out_dtype=torch.float32)
         ids, weights = ops.route_topk(z, self.correction, self.scale, self.top)
-        return ops.routed_experts(x, ids, weights, self.w_up, self.w_down, "gelu_erf")
+        return ops.routed_experts(x, ids, weights, self.w_up, self.w_down, "gelu_erf", combine=combine)
+
+    sums_in_residual = True     # forward32(x, combine=False) is there
 
     def forward(self, x, residual=None):
         y = self.forward32(x)

@@ -108,7 +108,8 @@ class PreNormStream32(Arrangement):
         y = self.mixer.forward32(self.norm_a(x), ctx.of("mixer"))
         if self.ffn is not None:
             x32, _, h = self._sum(x32, y, norm=self.norm_f)
-            y = self.ffn.forward32(h)
+            # (a routed feed-forward leaves the sum over a row's chosen experts to the residual sum's kernel)
+            y = self.ffn.forward32(h, combine=False) if getattr(self.ffn, "sums_in_residual", False) else self.ffn.forward32(h)
         # the block's last sum also applies the norm that reads its result next, where that norm can be fused
         after = ctx.next_norm if hasattr(ctx.next_norm, "fused") else None
         if self.side is None:
