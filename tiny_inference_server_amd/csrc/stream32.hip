@@ -184,13 +184,24 @@ __global__ __launch_bounds__(S32_THREADS) void residual_norm_kernel(
   const long r = blockIdx.x;
   constexpr int P = PER > 0 ? PER : 1;
   const bool y = y_in != nullptr || cs.ids != nullptr;        // whether there is a branch at all
+  // a row's choices and their weights, once for all its columns (up to 64 choices; beyond, from memory every time)
+  __shared__ int chosen_id[64];
+  __shared__ float chosen_w[64];
+  const bool kept = cs.ids && cs.top <= 64;
+  if (kept) {
+    if (threadIdx.x < cs.top) {
+      chosen_id[threadIdx.x] = cs.ids[r * cs.top + threadIdx.x];
+      chosen_w[threadIdx.x] = cs.weights[r * cs.top + threadIdx.x];
+    }
+    __syncthreads();
+  }
   auto y_at = [&](int c) {
     if (!cs.ids) return y_in[r * ldy + c];
     float v = 0.f;
     for (int k = 0; k < cs.top; ++k) {
-      const float w = cs.weights[r * cs.top + k];
-      v += w * (cs.ids[r * cs.top + k] < cs.n_experts ? y_in[(r * cs.top + k) * ldy + c]
-                                                        : to_f(static_cast<const T*>(cs.rows)[r * cs.ldr + c]));
+      const int e = kept ? chosen_id[k] : cs.ids[r * cs.top + k];
+      const float w = kept ? chosen_w[k] : cs.weights[r * cs.top + k];
+      v += w * (e < cs.n_experts ? y_in[(r * cs.top + k) * ldy + c] : to_f(static_cast<const T*>(cs.rows)[r * cs.ldr + c]));
     }
     return v;
   };
